@@ -93,6 +93,19 @@ int moe_sort_by_expert(const void* expert_idx, int in64, int64_t R, int E, int b
                        void* sorted_pos, int out64, void* counts, void* offsets, void* padded_blocks,
                        int64_t padded_cap, int32_t* num_padded, int32_t* inv, void* workspace, size_t workspace_bytes,
                        void* stream);
+/* moe_sort_by_expert for callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc).  No counterpart in the reference.  Same arguments, results and kernels as
+ * moe_sort_by_expert minus the workspace: the per-chunk histograms live in a static device array of the library,
+ * moe_sort_static_max_bytes() = 1 MiB per GPU, held until the process ends.  Limit: moe_sort_workspace_bytes(R, E)
+ * = (ceil(R / 512) * E + 4) * 4 bytes must fit in it (e.g. R <= 16.7 M assignments at E = 8), otherwise
+ * MOE_ERR_WORKSPACE and nothing is enqueued.  Calls no hipMalloc / hipFree and no allocating routine.  All calls on
+ * one GPU share that GPU's array: calls that overlap on one GPU (two streams, two threads) race; calls on one stream
+ * are ordered.  The first call on a device looks the array's address up (hipGetSymbolAddress) -- make that call
+ * outside stream capture. */
+size_t moe_sort_static_max_bytes(void);
+int moe_sort_by_expert_static(const void* expert_idx, int in64, int64_t R, int E, int block_m, void* sorted_expert,
+                              void* sorted_pos, int out64, void* counts, void* offsets, void* padded_blocks,
+                              int64_t padded_cap, int32_t* num_padded, int32_t* inv, void* stream);
 /* offsets[e] = #{i : sorted_expert[i] <= e}  (the expert_offsets consumed at ops.py:315-319) */
 int moe_expert_offsets(const void* sorted_expert, int in64, int64_t R, int E, void* offsets, int out64, void* stream);
 /* padded_block_indices from the inclusive offsets (ops.py:39-51) */

@@ -30,6 +30,8 @@ _SIGNATURES = {
     "moe_gemm_debug_plan": ("i", "piilllii" + "pp"),
     "moe_sort_workspace_bytes": ("z", "li"),
     "moe_sort_by_expert": ("i", "piliippippplpppzp"),
+    "moe_sort_static_max_bytes": ("z", ""),
+    "moe_sort_by_expert_static": ("i", "piliippippplppp"),
     "moe_expert_offsets": ("i", "pilipip"),
     "moe_padded_block_indices": ("i", "piiipilpp"),
     "moe_scatter2scatter_workspace_bytes": ("z", "lilli"),

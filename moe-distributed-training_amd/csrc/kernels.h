@@ -127,6 +127,11 @@ size_t moe_sort_ws_bytes(int64_t R, int E);
 int moe_launch_sort(const void* expert_idx, int in64, int64_t R, int E, int block_m, void* sorted_expert,
                     void* sorted_pos, int out64, void* counts, void* offsets, void* padded_blocks, int64_t padded_cap,
                     int32_t* num_padded, int32_t* inv, void* workspace, size_t workspace_bytes, hipStream_t stream);
+// the same sort with its per-chunk histograms in a static device array of the library (no workspace, no allocation)
+size_t moe_sort_static_capacity_bytes();
+int moe_launch_sort_static(const void* expert_idx, int in64, int64_t R, int E, int block_m, void* sorted_expert,
+                           void* sorted_pos, int out64, void* counts, void* offsets, void* padded_blocks,
+                           int64_t padded_cap, int32_t* num_padded, int32_t* inv, hipStream_t stream);
 int moe_launch_offsets_from_sorted(const void* sorted_expert, int in64, int64_t R, int E, void* offsets, int out64,
                                    hipStream_t stream);
 int moe_launch_padded_blocks(const void* offsets, int off64, int E, int block_m, void* padded_blocks, int out64,

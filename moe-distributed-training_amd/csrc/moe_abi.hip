@@ -153,6 +153,18 @@ int moe_sort_by_expert(const void* expert_idx, int in64, int64_t R, int E, int b
                            padded_blocks, padded_cap, num_padded, inv, workspace, workspace_bytes, st);
 }
 
+size_t moe_sort_static_max_bytes(void) { return moe_sort_static_capacity_bytes(); }
+
+int moe_sort_by_expert_static(const void* expert_idx, int in64, int64_t R, int E, int block_m, void* sorted_expert,
+                              void* sorted_pos, int out64, void* counts, void* offsets, void* padded_blocks,
+                              int64_t padded_cap, int32_t* num_padded, int32_t* inv, void* stream)
+{
+    if (R > 0 && (!expert_idx || !sorted_expert || !sorted_pos)) return MOE_ERR_BAD_ARG;
+    if (R >= (int64_t)1 << 31) return MOE_ERR_UNSUPPORTED;
+    return moe_launch_sort_static(expert_idx, in64, R, E, block_m, sorted_expert, sorted_pos, out64, counts, offsets,
+                                  padded_blocks, padded_cap, num_padded, inv, S(stream));
+}
+
 int moe_expert_offsets(const void* sorted_expert, int in64, int64_t R, int E, void* offsets, int out64, void* stream)
 {
     if ((R > 0 && !sorted_expert) || !offsets || E < 1) return MOE_ERR_BAD_ARG;

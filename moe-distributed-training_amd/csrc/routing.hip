@@ -4,6 +4,7 @@
 // LDS/global atomics are only used for integer counts whose final value is order independent).
 #include "common.h"
 #include "kernels.h"
+#include <mutex>
 
 namespace {
 
@@ -490,6 +491,50 @@ int moe_launch_sort(const void* expert_idx, int in64, int64_t R, int E, int bloc
         hipLaunchKernelGGL(sort_scatter_kernel, dim3(nblk), dim3(SORT_THREADS), (SORT_THREADS / 64) * E * sizeof(int32_t),
                            stream, expert_idx, in64, R, E, hist, sorted_expert, sorted_pos, out64, inv);
     return moe_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// The same sort for callers that cannot allocate or pass a workspace: the per-chunk histograms live in a static
+// device array (each GPU the library runs on holds its own copy at its own address until the process ends).
+// Every call on a GPU shares that GPU's array: calls that overlap on one GPU race.  Nothing in it has to start at
+// zero -- the histogram launch writes every cell the later launches read.
+// ---------------------------------------------------------------------------------------------------------
+constexpr int64_t SORT_STATIC_INTS = 262144;   // 1 MiB: ceil(R / 512) * E + 4 cells at most
+static __device__ __align__(256) int32_t scratch[SORT_STATIC_INTS];
+
+constexpr int SORT_STATIC_MAX_DEVICES = 64;
+static std::mutex g_scratch_mu;
+static int32_t* g_scratch_ptr[SORT_STATIC_MAX_DEVICES] = {};
+
+// Device address of `scratch` on the current device.  In host code the array's name is only a handle: the address a
+// kernel may use comes from hipGetSymbolAddress, once per device with that device current.
+static int sort_static_scratch(int32_t** out)
+{
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= SORT_STATIC_MAX_DEVICES) return MOE_ERR_LAUNCH;
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return MOE_ERR_LAUNCH;
+        g_scratch_ptr[dev] = (int32_t*)p;
+    }
+    *out = g_scratch_ptr[dev];
+    return MOE_OK;
+}
+
+size_t moe_sort_static_capacity_bytes() { return (size_t)SORT_STATIC_INTS * sizeof(int32_t); }
+
+int moe_launch_sort_static(const void* expert_idx, int in64, int64_t R, int E, int block_m, void* sorted_expert,
+                           void* sorted_pos, int out64, void* counts, void* offsets, void* padded_blocks,
+                           int64_t padded_cap, int32_t* num_padded, int32_t* inv, hipStream_t stream)
+{
+    if (E < 1 || E > 4096 || R < 0 || block_m < 1) return MOE_ERR_BAD_ARG;
+    if (moe_sort_ws_bytes(R, E) > moe_sort_static_capacity_bytes()) return MOE_ERR_WORKSPACE;
+    int32_t* ptr = nullptr;
+    const int rc = sort_static_scratch(&ptr);
+    if (rc != MOE_OK) return rc;
+    return moe_launch_sort(expert_idx, in64, R, E, block_m, sorted_expert, sorted_pos, out64, counts, offsets,
+                           padded_blocks, padded_cap, num_padded, inv, ptr, moe_sort_static_capacity_bytes(), stream);
 }
 
 int moe_launch_offsets_from_sorted(const void* sorted_expert, int in64, int64_t R, int E, void* offsets, int out64,
