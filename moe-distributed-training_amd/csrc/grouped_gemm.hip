@@ -19,6 +19,9 @@
 #include "kernels.h"
 #include <type_traits>
 
+#ifndef SK_ORDER
+#define SK_ORDER __ATOMIC_ACQ_REL
+#endif
 constexpr int NXCD_HOST = 8;
 static int moe_num_cus()
 {
@@ -534,7 +537,7 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
             }
         __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave's stores are acknowledged
         __syncthreads();                      // ... and every wave's: the partial is visible
-        if (tid == 0) *s_arrival = __hip_atomic_fetch_add(&p.sk_counters[ti], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (tid == 0) *s_arrival = __hip_atomic_fetch_add(&p.sk_counters[ti], 1, SK_ORDER, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
         if (*s_arrival != nparts - 1) return;
         if (tid == 0) __hip_atomic_store(&p.sk_counters[ti], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // clean for the next launch

@@ -7,9 +7,21 @@ import torch
 pytestmark = pytest.mark.gpu
 
 
-def rel(a, b):
-    b = b.float()
-    return float((a.detach().float().cpu() - b.detach()).abs().max() / b.detach().abs().max().clamp_min(1e-20))
+from _metrics import rel, rel_per_expert
+
+
+# Groups of one to a few rows, measured on their own scale: an adapter gradient is then a product of values that each
+# went through bf16 storage (dh, gate / up, dgate / dup, the low-rank interim, the result: five roundings of up to 2^-9
+# in a row, as in the reference, whose tensors are bf16 too) with no sum over many rows to average them out, so the
+# worst element of the worst slice sits at about 1 %, not well below it as for groups of hundreds of rows.
+TINY_GROUP_TOL = 1.5e-2
+
+
+def check_expert_grads(got, want, what, tol=1e-2):
+    """Adapter / weight gradients (first dimension = expert): each expert's slice against its own scale; the RMS
+    figure beside the maximum catches an error spread thinly over a slice."""
+    mx, rms = rel_per_expert(got, want, with_rms=True)
+    assert mx < tol and rms < tol, f"{what}: per-expert max rel err {mx:.4g}, rms rel err {rms:.4g}"
 
 
 def _make(T, d, f, E, r, dtype, seed=0, lora_std=0.02):
@@ -65,11 +77,11 @@ def test_layer_fwd_bwd_bf16(dev, oracle, T, d, f, E, r):
         ref2.backward(dout.float())
         for n, a, b in zip(("w1", "w2", "w3"), wd, wo):
             assert a.grad is not None and a.grad.shape == b.grad.shape
-            assert rel(a.grad, b.grad) < 1e-2, f"dW {n}"
+            check_expert_grads(a.grad, b.grad, f"dW {n}")
     if lora is not None:
         for n in ("w1", "w3", "w2"):
-            assert rel(lt[n][0].grad, lo[n][0].grad) < 1e-2, f"dA {n}"
-            assert rel(lt[n][1].grad, lo[n][1].grad) < 1e-2, f"dB {n}"
+            check_expert_grads(lt[n][0].grad, lo[n][0].grad, f"dA {n}")
+            check_expert_grads(lt[n][1].grad, lo[n][1].grad, f"dB {n}")
     # run-to-run determinism (activation checkpointing replays the forward inside backward)
     out2, _, ei2 = moe.moe_layer_forward(xg, wg.to(dev), wd[0], wd[1], wd[2], k, views, alpha)
     assert torch.equal(out2, out) and torch.equal(ei2, ei)
@@ -100,11 +112,11 @@ def test_layer_many_experts_and_wider_top_k(dev, oracle, E, k, r):
         ref2, _ = oracle.moe_block(x.float(), wg.float(), wo[0], wo[1], wo[2], k, None, alpha)
         ref2.backward(dout.float())
         for n, a, b in zip(("w1", "w2", "w3"), wd, wo):
-            assert rel(a.grad, b.grad) < 1e-2, f"dW {n}"
+            check_expert_grads(a.grad, b.grad, f"dW {n}", TINY_GROUP_TOL)
     else:
         for n in ("w1", "w3", "w2"):
-            assert rel(lt[n][0].grad, lo[n][0].grad) < 1e-2, f"dA {n}"
-            assert rel(lt[n][1].grad, lo[n][1].grad) < 1e-2, f"dB {n}"
+            check_expert_grads(lt[n][0].grad, lo[n][0].grad, f"dA {n}", TINY_GROUP_TOL)
+            check_expert_grads(lt[n][1].grad, lo[n][1].grad, f"dB {n}", TINY_GROUP_TOL)
 
 
 @pytest.mark.parametrize("r", [32, 24, 48])
@@ -126,8 +138,8 @@ def test_layer_rank_above_16_adapters(dev, oracle, r):
     assert torch.equal(ei.cpu().long(), aux["indices"])
     assert rel(out, ref) < 1e-2 and rel(xg.grad, xo.grad) < 1e-2
     for n in ("w1", "w3", "w2"):
-        assert rel(lt[n][0].grad, lo[n][0].grad) < 1e-2, f"dA {n}"
-        assert rel(lt[n][1].grad, lo[n][1].grad) < 1e-2, f"dB {n}"
+        check_expert_grads(lt[n][0].grad, lo[n][0].grad, f"dA {n}")
+        check_expert_grads(lt[n][1].grad, lo[n][1].grad, f"dB {n}")
 
 
 def test_layer_expert_weights_output_carries_grad(dev, oracle):
@@ -260,7 +272,7 @@ def test_fused_mlp_full_finetune_weight_grads(dev, oracle, use_gates):
     out.backward(dout.to(dev))
     assert rel(out, ref) < 1e-2 and rel(xg.grad, xo.grad) < 1e-2
     for n, a, b in zip(("w1", "w2", "w3"), wd, wo):
-        assert rel(a.grad, b.grad) < 1e-2, f"dW {n}"
+        check_expert_grads(a.grad, b.grad, f"dW {n}")
 
 
 def test_block_module_returns_hidden_and_none(dev):
@@ -304,8 +316,78 @@ def test_mixtral_shape_full_size(dev, oracle):
     assert flips == 0, f"{flips} tokens routed differently from the fp32 oracle"
     assert rel(out, ref) < 1e-2 and rel(xg.grad, xo.grad) < 1e-2
     for n in ("w1", "w3", "w2"):
-        assert rel(lt[n][0].grad, lo[n][0].grad) < 1e-2, f"dA {n}"
-        assert rel(lt[n][1].grad, lo[n][1].grad) < 1e-2, f"dB {n}"
+        check_expert_grads(lt[n][0].grad, lo[n][0].grad, f"dA {n}")
+        check_expert_grads(lt[n][1].grad, lo[n][1].grad, f"dB {n}")
+
+
+@pytest.mark.slow
+def test_mixtral_shape_skewed_routing_full_gradients(dev, oracle):
+    """BASELINE configs[3]'s routing (Zipf s=1.2 logit offsets: the top expert takes ~40 % of the assignments, the
+    last ones are near-empty) at the real d, f with LoRA, T=4096, fwd+bwd: out, dX and all six adapter gradients
+    against the fp32 oracle, every expert's slice on its own scale -- a ragged tail whose rows were dropped, or a
+    near-empty group that was mishandled, cannot hide behind the large groups."""
+    import moe_distributed_training_amd as moe
+    T, d, f, E, k, r, alpha = 4096, 4096, 14336, 8, 2, 16, 32.0
+    g = torch.Generator(device=dev).manual_seed(4)
+    rn = lambda *s, std=1.0: (torch.randn(*s, generator=g, device=dev) * std).bfloat16()
+    x, wg = rn(T, d), rn(E, d, std=0.02)
+    pmf = torch.tensor([1.0 / (i + 1) ** 1.2 for i in range(E)]); pmf /= pmf.sum()
+    x[:, 0] = 1.0
+    wg[:, 0] = (2.2 * torch.log(pmf)).bfloat16().to(dev)
+    w1, w2, w3 = rn(E, f, d, std=0.02), rn(E, f, d, std=0.02), rn(E, f, d, std=0.02)
+    lora = {"w1": (rn(E, d, r, std=0.02), rn(E, r, f, std=0.02)), "w3": (rn(E, d, r, std=0.02), rn(E, r, f, std=0.02)),
+            "w2": (rn(E, f, r, std=0.02), rn(E, r, d, std=0.02))}
+    dout = rn(T, d)
+    lt, views = _views({n: (a.cpu(), b.cpu()) for n, (a, b) in lora.items()}, dev)
+    xg = x.clone().requires_grad_(True)
+    out, ew, ei = moe.moe_layer_forward(xg, wg, w1, w2, w3, k, views, alpha)
+    out.backward(dout)
+    torch.cuda.synchronize()
+    torch.set_num_threads(16)
+    xo = x.float().cpu().requires_grad_(True)
+    lo = {n: (a.float().cpu().requires_grad_(True), b.float().cpu().requires_grad_(True)) for n, (a, b) in lora.items()}
+    ref, aux = oracle.moe_block(xo, wg.float().cpu(), w1.float().cpu(), w2.float().cpu(), w3.float().cpu(), k, lo, alpha)
+    ref.backward(dout.float().cpu())
+    assert torch.equal(ei.cpu().long(), aux["indices"])
+    counts = torch.bincount(aux["indices"].flatten(), minlength=E)
+    assert counts.max() > 0.3 * T * k and counts.min() < 0.05 * T * k, counts.tolist()
+    assert rel(out, ref) < 1e-2 and rel(xg.grad, xo.grad) < 1e-2
+    for n in ("w1", "w3", "w2"):
+        check_expert_grads(lt[n][0].grad, lo[n][0].grad, f"dA {n} counts={counts.tolist()}")
+        check_expert_grads(lt[n][1].grad, lo[n][1].grad, f"dB {n} counts={counts.tolist()}")
+
+
+@pytest.mark.slow
+def test_ep_share_full_size(dev, oracle):
+    """BASELINE configs[4] at its real size: one expert-parallel rank's share, 2 resident experts, 8192 pre-dispatched
+    rows (group sizes from a 0.55 / 0.45 draw, arrival order a permutation), fan-out 1, LoRA r=16, fwd+bwd, against the
+    fp32 oracle (two experts over 8 XCDs, ~18 row tiles each: the tile plan of few, large groups)."""
+    import moe_distributed_training_amd as moe
+    d, f, r, alpha, E, R = 4096, 14336, 16, 32.0, 2, 8192
+    g = torch.Generator(device=dev).manual_seed(6)
+    rn = lambda *s, std=1.0: (torch.randn(*s, generator=g, device=dev) * std).bfloat16()
+    w1, w2, w3 = rn(E, f, d, std=0.02), rn(E, f, d, std=0.02), rn(E, f, d, std=0.02)
+    lora = {"w1": (rn(E, d, r, std=0.02), rn(E, r, f, std=0.02)), "w3": (rn(E, d, r, std=0.02), rn(E, r, f, std=0.02)),
+            "w2": (rn(E, f, r, std=0.02), rn(E, r, d, std=0.02))}
+    xr, dy = rn(R, d), rn(R, d)
+    e_of_row = (torch.rand(R, generator=torch.Generator().manual_seed(7)) > 0.55).long()
+    sei, ssi = oracle.flatten_and_sort(e_of_row)
+    eo = torch.bincount(sei, minlength=E).cumsum(0)
+    lt, views = _views({n: (a.cpu(), b.cpu()) for n, (a, b) in lora.items()}, dev)
+    xg = xr.clone().requires_grad_(True)
+    y = moe.fused_expert_mlp(xg, w1, w2, w3, 1, ssi.int().to(dev), eo.int().to(dev), views, alpha)
+    y.backward(dy)
+    torch.cuda.synchronize()
+    torch.set_num_threads(16)
+    xo = xr.float().cpu().requires_grad_(True)
+    lo = {n: (a.float().cpu().requires_grad_(True), b.float().cpu().requires_grad_(True)) for n, (a, b) in lora.items()}
+    ref, _ = oracle.moe_block(xo, None, w1.float().cpu(), w2.float().cpu(), w3.float().cpu(), 1, lo, alpha,
+                              routing=(torch.ones(R, 1), e_of_row[:, None]))
+    ref.backward(dy.float().cpu())
+    assert rel(y, ref) < 1e-2 and rel(xg.grad, xo.grad) < 1e-2
+    for n in ("w1", "w3", "w2"):
+        check_expert_grads(lt[n][0].grad, lo[n][0].grad, f"dA {n}")
+        check_expert_grads(lt[n][1].grad, lo[n][1].grad, f"dB {n}")
 
 
 @pytest.mark.slow
@@ -338,7 +420,7 @@ def test_skewed_routing_and_ep_share(dev, oracle):
     ref.backward(dy.float().cpu())
     assert rel(y, ref) < 1e-2 and rel(xg.grad, xo.grad) < 1e-2
     for n in ("w1", "w3", "w2"):
-        assert rel(lt[n][0].grad, lo[n][0].grad) < 1e-2 and rel(lt[n][1].grad, lo[n][1].grad) < 1e-2
+        check_expert_grads(lt[n][0].grad, lo[n][0].grad, f"dA {n}"); check_expert_grads(lt[n][1].grad, lo[n][1].grad, f"dB {n}")
     # --- skewed routing through the whole layer with the same two experts' weights replicated to E=8 views
     E8 = 8
     w1e, w2e, w3e = (t.repeat(4, 1, 1) for t in (w1, w2, w3))
@@ -387,11 +469,11 @@ def test_skewed_full_size_properties(dev, oracle):
         xg = x.clone().requires_grad_(True)
         out, ew, ei = moe.moe_layer_forward(xg, wg, w1, w2, w3, k, views, alpha)
         out.backward(dout)
-        return out.detach(), ei, xg.grad, {n: (lt[n][0].grad, lt[n][1].grad) for n in lt}
+        return out.detach(), ei, xg.grad, {n: (lt[n][0].grad, lt[n][1].grad) for n in lt}, ew.detach()
 
-    out, ei, dx1, g1 = run(d1)
-    _, _, dx2, g2 = run(d2)
-    _, _, dx3, g3 = run((d1.float() + d2.float()).bfloat16())
+    out, ei, dx1, g1, ew = run(d1)
+    _, _, dx2, g2, _ = run(d2)
+    _, _, dx3, g3, _ = run((d1.float() + d2.float()).bfloat16())
     counts = torch.bincount(ei.flatten().cpu().long(), minlength=E)
     assert int(counts.sum()) == T * k and counts.max() > 0.3 * T * k and counts.min() < 0.05 * T * k   # really skewed
     rt = router.route_and_sort(x, wg, k)
@@ -411,6 +493,20 @@ def test_skewed_full_size_properties(dev, oracle):
     ref.backward(d1[sl].float().cpu())
     assert torch.equal(ei[sl].cpu().long(), aux["indices"])
     assert rel(out[sl], ref) < 1e-2 and rel(dx1[sl], xo.grad) < 1e-2
+    # (4) adapter gradients of single experts against the oracle: an expert's dA / dB depend only on the rows routed to
+    # it, so the oracle run on those tokens alone (one assignment each, the layer's own routing weight) gives them.  The
+    # smallest group (near-empty) and a mid-sized one; the largest is covered at T=4096 with the same routing law.
+    ewc, eic = ew.float().cpu(), ei.cpu().long()
+    order = torch.argsort(counts)
+    for e in (int(order[0]), int(order[E // 2])):
+        tok, slot = torch.where(eic == e)
+        loe = {n: (a.float().cpu().requires_grad_(True), b.float().cpu().requires_grad_(True)) for n, (a, b) in lora.items()}
+        refe, _ = oracle.moe_block(x[tok.to(dev)].float().cpu(), None, w1.float().cpu(), w2.float().cpu(), w3.float().cpu(), 1, loe, alpha,
+                                   routing=(ewc[tok, slot][:, None], torch.full((tok.numel(), 1), e)))
+        refe.backward(d1[tok.to(dev)].float().cpu())
+        for n in ("w1", "w3", "w2"):
+            for j, nm in ((0, "dA"), (1, "dB")):
+                check_expert_grads(g1[n][j][e:e + 1], loe[n][j].grad[e:e + 1], f"{nm} {n} expert {e} ({tok.numel()} rows)")
 
 
 def test_step_captures_into_a_graph_and_replays_bit_identically(dev):
@@ -481,7 +577,7 @@ def test_tiny_and_empty_batches(dev, oracle, T, r):
     assert rel(out, ref) < 1e-2 and rel(xg.grad, xo.grad) < 1e-2
     if lora is not None:
         for n in ("w1", "w3", "w2"):   # experts that received no row get exact zeros
-            assert rel(lt[n][0].grad, lo[n][0].grad) < 1e-2 and rel(lt[n][1].grad, lo[n][1].grad) < 1e-2
+            check_expert_grads(lt[n][0].grad, lo[n][0].grad, f"dA {n}", TINY_GROUP_TOL); check_expert_grads(lt[n][1].grad, lo[n][1].grad, f"dB {n}", TINY_GROUP_TOL)
             unused = [e for e in range(E) if e not in aux["indices"].flatten().tolist()]
             assert float(lt[n][0].grad[unused].abs().max()) == 0.0 and float(lt[n][1].grad[unused].abs().max()) == 0.0
 
@@ -516,5 +612,5 @@ def test_layer_seeded_shape_sweep(dev, oracle, seed):
     assert rel(out, ref) < 1e-2 and rel(xg.grad, xo.grad) < 1e-2, case
     if lora is not None:
         for n in ("w1", "w3", "w2"):
-            assert rel(lt[n][0].grad, lo[n][0].grad) < 1e-2, f"dA {n} {case}"
-            assert rel(lt[n][1].grad, lo[n][1].grad) < 1e-2, f"dB {n} {case}"
+            check_expert_grads(lt[n][0].grad, lo[n][0].grad, f"dA {n} {case}", TINY_GROUP_TOL)
+            check_expert_grads(lt[n][1].grad, lo[n][1].grad, f"dB {n} {case}", TINY_GROUP_TOL)
