@@ -24,13 +24,24 @@ sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
 PEAK_HBM_GBS = 8000.0
-# HBM-side bytes per launch of the grouped GEMM stages for the default workload, from rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE with the calibration factors recorded in profiles/grouped_gemm_hbm_traffic_pmc.txt (counters cannot be read
-# from inside this process; the figures are refreshed whenever that profile is)
-MEASURED_TRAFFIC_BYTES = {
-    "mixtral_fwd_bwd_lora": {"fwd.gemm_w1w3_swiglu": 4.27e9, "bwd.gemm_dh_swiglu_bwd": 2.77e9,
-                             "fwd.gemm_w2": 2.25e9, "bwd.gemm_dx_w1w3": 4.53e9},
-}
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "grouped_gemm_hbm_traffic_pmc.txt")
+
+
+def measured_traffic_bytes(path=TRAFFIC_PROFILE):
+    """HBM-side bytes per launch of the grouped GEMM stages, read from the committed rocprofv3 --pmc FETCH_SIZE /
+    WRITE_SIZE summary (counters cannot be read from inside this process): its lines
+    `traffic_bytes <workload> <stage> <bytes>` carry the calibrated figures."""
+    out = {}
+    try:
+        with open(path) as fh:
+            for line in fh:
+                parts = line.split()
+                if len(parts) == 4 and parts[0] == "traffic_bytes":
+                    out.setdefault(parts[1], {})[parts[2]] = float(parts[3])
+    except OSError:
+        pass
+    return out
+
 
 WORKLOADS = {
     # name: (T, d, f, E, k, rank, backward, skew, description)
@@ -42,15 +53,22 @@ WORKLOADS = {
                         desc="Mixtral-8x7B MoE layer forward, T=4096, bf16, top-2 (BASELINE configs[1])"),
     "mixtral_fwd_bwd_full": dict(T=4096, d=4096, f=14336, E=8, k=2, r=0, bwd=True, skew=False, train_base=True,
                                  desc="Mixtral-8x7B MoE layer fwd+bwd, T=4096, bf16, top-2, full fine-tuning (expert weights take gradients)"),
+    "ep_share_fwd_bwd_lora": dict(T=8192, d=4096, f=14336, E=2, k=1, r=16, bwd=True, skew=False, ep_share=True,
+                                  desc="one expert-parallel rank's share: 2 resident experts, 8192 pre-dispatched rows (0.55 / 0.45), "
+                                       "bf16, LoRA r=16, fwd+bwd, no router / combine (BASELINE configs[4])"),
+    "tiny_fp32_fwd": dict(T=256, d=128, f=256, E=4, k=2, r=0, bwd=False, skew=False, dtype="fp32",
+                          desc="tiny MoE MLP, T=256, d=128, f=256, E=4, top-2, fp32, forward (BASELINE configs[0], the CPU-runnable case)"),
     "skewed_fwd_bwd_lora": dict(T=16384, d=4096, f=14336, E=8, k=2, r=16, bwd=True, skew=True,
                                 desc="Zipf(1.2)-skewed routing, T=16384, fwd+bwd, LoRA r=16 (BASELINE configs[3])"),
 }
 
 
-def flops(T, d, f, E, k, r, bwd, train_base=False):
+def flops(T, d, f, E, k, r, bwd, train_base=False, ep_share=False):
+    """Algorithmic FLOP of one step.  ep_share: rows arrive dispatched (T rows, one assignment each), the router runs
+    on the other side of the exchange and is not counted."""
     R = T * k
     base = 6 * R * d * f
-    router = 2 * T * d * E
+    router = 0 if ep_share else 2 * T * d * E
     lora_fwd = 6 * R * r * (d + f)
     total = base + router + lora_fwd
     if bwd:
@@ -64,7 +82,7 @@ def make_inputs(cfg, dev, seed=0):
     import torch
     g = torch.Generator(device=dev).manual_seed(seed)
     T, d, f, E, r = cfg["T"], cfg["d"], cfg["f"], cfg["E"], cfg["r"]
-    bf = torch.bfloat16
+    bf = torch.float32 if cfg.get("dtype") == "fp32" else torch.bfloat16
 
     def rn(*shape, std=1.0):
         return (torch.randn(*shape, generator=g, device=dev, dtype=torch.float32) * std).to(bf)
@@ -73,7 +91,6 @@ def make_inputs(cfg, dev, seed=0):
     wg = rn(E, d, std=0.02)
     if cfg["skew"]:
         # per-expert logit offset ~ log Zipf(s=1.2) pmf, folded into the router weight along one input direction
-        import math
         pmf = torch.tensor([1.0 / (i + 1) ** 1.2 for i in range(E)])
         pmf = pmf / pmf.sum()
         bias = (2.2 * torch.log(pmf)).to(dev)
@@ -88,6 +105,19 @@ def make_inputs(cfg, dev, seed=0):
     return x, wg, w1, w2, w3, lora, dout
 
 
+def ep_share_routing(cfg, dev, seed=1):
+    """The local expert of each pre-dispatched row (a multinomial draw, 0.55 / 0.45 over the two resident experts; rows
+    arrive in exchange order, i.e. the grouped order is a permutation of them) and what the rank's local re-sort hands
+    to the kernels: sorted positions and inclusive expert offsets."""
+    import torch
+    from moe_distributed_training_amd.megablocks_utils.router import sort_assignments
+    g = torch.Generator().manual_seed(seed)
+    p = torch.tensor([0.55, 0.45] if cfg["E"] == 2 else [1.0 / cfg["E"]] * cfg["E"])
+    e_of_row = torch.multinomial(p, cfg["T"], replacement=True, generator=g).to(dev)
+    _sei, ssi, _counts, offsets, _inv = sort_assignments(e_of_row.int(), cfg["E"])
+    return e_of_row, ssi, offsets
+
+
 def read_profile(lib):
     n = lib.moe_profile_count()
     buf = ctypes.create_string_buffer(64)
@@ -99,8 +129,10 @@ def read_profile(lib):
     return out
 
 
-def cpu_baseline(cfg, x, wg, w1, w2, w3, lora, dout, budget_tokens):
-    """fp32 CPU oracle (per-expert loop + index_add, autograd backward) on the first `budget_tokens` tokens."""
+def cpu_baseline(cfg, x, wg, w1, w2, w3, lora, dout, budget_tokens, e_of_row=None):
+    """fp32 CPU oracle (per-expert loop + index_add, autograd backward) on the first `budget_tokens` tokens: one
+    untimed warm-up pass, then the median of 3 timed passes (5 for the tiny configuration)."""
+    import statistics
     import torch
     from oracle import moe_oracle as oracle
     cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
@@ -118,16 +150,33 @@ def cpu_baseline(cfg, x, wg, w1, w2, w3, lora, dout, budget_tokens):
         lo = {"w1": (c["a1"], c["b1"]), "w3": (c["a3"], c["b3"]), "w2": (c["a2"], c["b2"])}
     ds = dout[:Ts].float().cpu()
     xs.requires_grad_(cfg["bwd"])
-    t0 = time.perf_counter()
-    with torch.set_grad_enabled(cfg["bwd"]):
-        out, _ = oracle.moe_block(xs, W[0], W[1], W[2], W[3], cfg["k"], lo, 32.0)
-        if cfg["bwd"]:
-            out.backward(ds)
-    dt = time.perf_counter() - t0
-    fl = flops(Ts, cfg["d"], cfg["f"], cfg["E"], cfg["k"], cfg["r"], cfg["bwd"], bool(cfg.get("train_base")))
+    routing = None
+    if e_of_row is not None:   # pre-dispatched rows: the expert of each row is given, weight 1
+        routing = (torch.ones(Ts, 1), e_of_row[:Ts].cpu().long()[:, None])
+
+    def one_pass():
+        t0 = time.perf_counter()
+        with torch.set_grad_enabled(cfg["bwd"]):
+            out, _ = oracle.moe_block(xs, None if routing else W[0], W[1], W[2], W[3], cfg["k"], lo, 32.0, routing=routing)
+            if cfg["bwd"]:
+                out.backward(ds)
+        return time.perf_counter() - t0
+
+    one_pass()
+    passes = 5 if cfg["T"] <= 1024 else 3
+    times = [one_pass() for _ in range(passes)]
+    dt = statistics.median(times)
+    fl = flops(Ts, cfg["d"], cfg["f"], cfg["E"], cfg["k"], cfg["r"], cfg["bwd"], bool(cfg.get("train_base")), bool(cfg.get("ep_share")))
+    cpu_model = "unknown CPU"
+    try:
+        with open("/proc/cpuinfo") as fh:
+            cpu_model = next(line.split(":", 1)[1].strip() for line in fh if line.startswith("model name"))
+    except (OSError, StopIteration):
+        pass
     return dict(value=fl / dt / 1e12, unit="TFLOP/s", cores=cores, kind="port",
-                sample=f"first {Ts} of {cfg['T']} tokens, one pass, fp32 torch oracle ({dt:.1f} s)",
-                tokens_per_s=Ts / dt)
+                sample=f"first {Ts} of {cfg['T']} {'rows' if cfg.get('ep_share') else 'tokens'}, fp32 torch oracle, 1 warm-up pass + median of "
+                       f"{passes} passes ({dt * 1e3:.1f} ms; all: {', '.join(f'{t * 1e3:.1f}' for t in times)} ms)",
+                tokens_per_s=Ts / dt, cpu=cpu_model)
 
 
 def library_gemm(torch, dev, R, d, f, launches=50):
@@ -181,17 +230,28 @@ def main():
     if train_base:
         for w in (w1, w2, w3):
             w.requires_grad_(True)
+    ep_share = bool(cfg.get("ep_share"))
+    e_of_row = ep_ssi = ep_offsets = None
+    if ep_share:
+        e_of_row, ep_ssi, ep_offsets = ep_share_routing(cfg, dev)
+
+    def clear_grads():
+        x.grad = None
+        if lora is not None:
+            for v in lora.values():
+                v.grad = None
+        if train_base:
+            w1.grad = w2.grad = w3.grad = None
 
     def step():
         with torch.set_grad_enabled(cfg["bwd"]):
-            out, ew, ei = moe.moe_layer_forward(x, wg, w1, w2, w3, cfg["k"], views, 32.0)
+            if ep_share:
+                # the rows are here already, one assignment each: expert MLP on the local experts, output back in arrival order
+                out = moe.fused_expert_mlp(x, w1, w2, w3, 1, ep_ssi, ep_offsets, views, 32.0)
+            else:
+                out, ew, ei = moe.moe_layer_forward(x, wg, w1, w2, w3, cfg["k"], views, 32.0)
             if cfg["bwd"]:
-                x.grad = None
-                if lora is not None:
-                    for v in lora.values():
-                        v.grad = None
-                if train_base:
-                    w1.grad = w2.grad = w3.grad = None
+                clear_grads()
                 out.backward(dout)
         return out
 
@@ -207,7 +267,7 @@ def main():
     prof = read_profile(lib)
     lib.moe_profile_enable(0)
 
-    fl = flops(cfg["T"], cfg["d"], cfg["f"], cfg["E"], cfg["k"], cfg["r"], cfg["bwd"], train_base)
+    fl = flops(cfg["T"], cfg["d"], cfg["f"], cfg["E"], cfg["k"], cfg["r"], cfg["bwd"], train_base, ep_share)
     tflops = fl / dt / 1e12
     stages = {k_: sum(v) / len(v) for k_, v in prof.items()}
     # dominant kernel: the grouped GEMM launches; FLOPs per launch are the algorithmic ones of that projection pair
@@ -216,25 +276,37 @@ def main():
                   "bwd.gemm_dh_swiglu_bwd": 2 * R * cfg["d"] * cfg["f"], "bwd.gemm_dx_w1w3": 4 * R * cfg["d"] * cfg["f"],
                   "bwd.group_bwd_w": 2 * R * cfg["d"] * cfg["f"]}
     gemm_stages = {k_: v for k_, v in stages.items() if k_ in gemm_flops}
-    dom = max(gemm_stages, key=gemm_stages.get)
-    ach = gemm_flops[dom] / (gemm_stages[dom] * 1e-3) / 1e12
-    per_step = {k_: len(prof[k_]) / args.steps for k_ in gemm_stages}       # launches per step (3 for the weight gradients)
-    gemm_ms = sum(gemm_stages[k_] * per_step[k_] for k_ in gemm_stages)
-    gemm_all = sum(gemm_flops[k_] * per_step[k_] for k_ in gemm_stages) / (gemm_ms * 1e-3) / 1e12
+    fp32 = cfg.get("dtype") == "fp32"
+    if gemm_stages:
+        dom = max(gemm_stages, key=gemm_stages.get)
+        ach = gemm_flops[dom] / (gemm_stages[dom] * 1e-3) / 1e12
+        per_step = {k_: len(prof[k_]) / args.steps for k_ in gemm_stages}       # launches per step (3 for the weight gradients)
+        gemm_ms = sum(gemm_stages[k_] * per_step[k_] for k_ in gemm_stages)
+        gemm_all = sum(gemm_flops[k_] * per_step[k_] for k_ in gemm_stages) / (gemm_ms * 1e-3) / 1e12
+        roofline = {"bound": "mfma", "kernel": f"{'grouped_xty_mfma_kernel' if dom == 'bwd.group_bwd_w' else 'grouped_gemm_mfma_kernel'} [{dom}]",
+                    "achieved": round(ach, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(ach / PEAK_BF16_TFLOPS, 4),
+                    "traffic": measured_traffic_bytes().get(args.workload, {}).get(dom), "launch_ms": round(gemm_stages[dom], 4),
+                    "all_gemm_launches_tflops": round(gemm_all, 2), "all_gemm_ms": round(gemm_ms, 4)}
+    else:
+        # fp32 runs on the generic (non matrix-core) kernels through the per-projection calls, which carry no stage timer: the
+        # whole step stands for the kernel, against the fp32 vector peak
+        peak = 157.3
+        roofline = {"bound": "mfma", "kernel": "generic_gemm_kernel (whole step: a few microseconds of work, launch bound)",
+                    "achieved": round(tflops, 4), "peak": peak, "unit": "TFLOP/s", "frac": round(tflops / peak, 6), "traffic": None}
+    what = ("fwd+bwd" if cfg["bwd"] else "fwd")
+    metric = "MoE-layer fwd+bwd TFLOP/s & % bf16 MFMA peak, Mixtral shape T=4096, 1 GPU" if args.workload == "mixtral_fwd_bwd_lora" \
+        else f"MoE-layer {what} TFLOP/s & % {'fp32' if fp32 else 'bf16 MFMA'} peak, workload {args.workload}, 1 GPU"
     result = {
-        "metric": "MoE-layer fwd+bwd TFLOP/s & % bf16 MFMA peak, Mixtral shape T=4096, 1 GPU",
-        "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "metric": metric,
+        "value": round(tflops, 4 if fp32 else 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(dt * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16", "data": "synthetic",
+        "dtype": "fp32" if fp32 else "bf16", "data": "synthetic",
         "config": {"workload": cfg["desc"], "tokens": cfg["T"], "d_model": cfg["d"], "d_ff": cfg["f"],
                    "experts": cfg["E"], "top_k": cfg["k"], "lora_rank": cfg["r"]},
         "tokens_per_s": round(cfg["T"] / dt, 1),
-        "frac_of_bf16_peak": round(tflops / PEAK_BF16_TFLOPS, 4),
+        "frac_of_bf16_peak": round(tflops / PEAK_BF16_TFLOPS, 6 if fp32 else 4),
         "algorithmic_flop_per_step": fl,
-        "roofline": {"bound": "mfma", "kernel": f"{'grouped_xty_mfma_kernel' if dom == 'bwd.group_bwd_w' else 'grouped_gemm_mfma_kernel'} [{dom}]", "achieved": round(ach, 2),
-                     "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(ach / PEAK_BF16_TFLOPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload, {}).get(dom), "launch_ms": round(gemm_stages[dom], 4),
-                     "all_gemm_launches_tflops": round(gemm_all, 2), "all_gemm_ms": round(gemm_ms, 4)},
+        "roofline": roofline,
         "stage_ms": {k_: round(v, 4) for k_, v in sorted(stages.items())},
     }
     # HBM-bound stages: algorithmic bytes (read activations once, write results once) over the measured launch times
@@ -249,11 +321,12 @@ def main():
         hbm["combine d_gates"] = (stages["rows.combine_dgates"], R * d_ * 2 + T_ * d_ * 2 + T_ * k_top * 4)
     result["hbm_stages"] = {n: {"ms": round(ms, 4), "bytes": b, "GB_per_s": round(b / (ms * 1e-3) / 1e9, 1),
                                 "frac_of_8TBps": round(b / (ms * 1e-3) / 8e12, 4)} for n, (ms, b) in hbm.items()}
-    result["library_gemm"] = library_gemm(torch, dev, R, cfg["d"], cfg["f"])
+    if not fp32:
+        result["library_gemm"] = library_gemm(torch, dev, R, cfg["d"], cfg["f"])
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(cfg, x.detach(), wg, w1, w2, w3,
                                               None if lora is None else {k_: v.detach() for k_, v in lora.items()},
-                                              dout, args.cpu_tokens)
+                                              dout, args.cpu_tokens, e_of_row)
         result["cpu_baseline"]["value"] = round(result["cpu_baseline"]["value"], 4)
         result["cpu_baseline"]["tokens_per_s"] = round(result["cpu_baseline"]["tokens_per_s"], 1)
     print(json.dumps(result))

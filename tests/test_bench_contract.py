@@ -27,3 +27,33 @@ def test_algorithmic_flops_of_the_workloads():
     assert abs(bench.flops(T, d, f, E, k, r, True) - 5.830e12) / 5.830e12 < 1e-3              # the figure quoted for the default workload
     for name, cfg in bench.WORKLOADS.items():
         assert {"T", "d", "f", "E", "k", "r", "bwd", "skew", "desc"} <= set(cfg), name
+
+
+def test_flops_of_the_expert_parallel_share_and_the_tiny_configuration():
+    sys.path.insert(0, ROOT)
+    import bench
+    d, f, r = 4096, 14336, 16
+    ep = bench.WORKLOADS["ep_share_fwd_bwd_lora"]
+    assert (ep["T"], ep["E"], ep["k"], ep["r"], ep["bwd"]) == (8192, 2, 1, 16, True)
+    R = 8192
+    # the Mixtral fwd+bwd+LoRA formula on 8192 rows, without the router (it runs on the other side of the exchange)
+    want = 12 * R * d * f + 24 * R * r * (d + f)
+    got = bench.flops(ep["T"], ep["d"], ep["f"], ep["E"], ep["k"], ep["r"], ep["bwd"], False, True)
+    assert got == want and abs(got - 5.830e12) / 5.830e12 < 1e-3
+    tiny = bench.WORKLOADS["tiny_fp32_fwd"]
+    assert (tiny["T"], tiny["d"], tiny["f"], tiny["E"], tiny["k"], tiny["dtype"], tiny["bwd"]) == (256, 128, 256, 4, 2, "fp32", False)
+    got = bench.flops(tiny["T"], tiny["d"], tiny["f"], tiny["E"], tiny["k"], 0, False)
+    assert got == 6 * 512 * 128 * 256 + 2 * 256 * 128 * 4 and abs(got - 1.007e8) / 1.007e8 < 5e-3
+
+
+def test_roofline_traffic_is_read_from_the_committed_profile():
+    sys.path.insert(0, ROOT)
+    import bench
+    t = bench.measured_traffic_bytes()
+    stages = t["mixtral_fwd_bwd_lora"]
+    assert set(stages) == {"fwd.gemm_w1w3_swiglu", "fwd.gemm_w2", "bwd.gemm_dx_w1w3", "bwd.gemm_dh_swiglu_bwd"}
+    assert all(1e9 < v < 1e10 for v in stages.values())
+    # the figures are the profile's own: each appears in its "scaled traffic per launch" table
+    text = open(bench.TRAFFIC_PROFILE).read()
+    for v in stages.values():
+        assert f"= {v / 1e9:.2f} GB" in text

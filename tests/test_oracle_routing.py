@@ -144,3 +144,14 @@ def test_router_switches_reduce_to_library_routines(oracle):
     assert torch.equal(ij, i_n) and torch.allclose(sj, s_n) and torch.allclose(wj, w_n)
     _, wu, iu = oracle.router_with_options(x, wg, 2, 1, uniform_expert_assignment=True)
     assert iu.flatten().tolist() == [j % 6 for j in range(80)] and torch.allclose(wu, w)
+
+
+def test_c_restatement_is_clean_under_asan_and_ubsan():
+    """The C restatement built with the host AddressSanitizer / UndefinedBehaviorSanitizer (`make -C oracle asan`) works
+    through exact-size buffers over edge sizes (no rows, one expert, block-size boundaries, skewed groups, ties in the
+    top-k) without a report and with every answer meeting its definition."""
+    import os, subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run(["make", "-B", "-C", os.path.join(root, "oracle"), "asan"], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+    assert "sanitizer run clean" in r.stdout and "ERROR" not in r.stderr and "runtime error" not in r.stderr
