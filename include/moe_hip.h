@@ -80,6 +80,14 @@ int moe_router_forward(const void* x, int64_t ldx, const void* wg, int64_t ldw, 
 int moe_router_topk_bwd(const float* dtopw, const float* topw, const int32_t* topi, const float* scores,
                         float* dlogits, int64_t ntok, int E, int k, int renorm, void* stream);
 
+/* gradient of the router weight: dwg[e][c] = sum_t dlogits[t][e] * x[t][c] (autograd of the F.linear at
+ * config_utils.py:262), from the fp32 dlogits with fp32 accumulation and a fixed summation order; dwg (E, d) in x's
+ * dtype.  The gradient with respect to the router's input, dlogits @ wg, is moe_combine with k = 0 and the dense
+ * tail (extra_coef = dlogits, extra_rows = wg). */
+size_t moe_router_weight_grad_workspace_bytes(int64_t ntok, int64_t d, int E);
+int moe_router_weight_grad(const void* x, int64_t ldx, const float* dlogits, void* dwg, int64_t ldo, int64_t ntok,
+                           int64_t d, int E, int dtype, void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- expert-grouped order: flatten_and_sort / histogram / cumsum / padded_block_indices ----------------------
  * Call sites: config_utils.py:114-118 (padded_block_indices), :131-132 (bin_ids, indices from megablocks'
  * stable radix sort), tests/test_scattermoe.py:84-85,161-163; block semantics scattermoe_utils/kernels/ops.py:39-51.
@@ -148,7 +156,8 @@ int moe_group_rows(const void* src, int64_t lds, void* out, int64_t ldo, const v
 
 /* ---- weighted combine: the gates bmm of parallel_linear_lora.py:30-35 / megablocks ops.scatter (config_utils.py:251)
  * out[t] = sum_j gates[t*k+j] * y[row(t,j)] (+ sum_e extra_coef[t][e] * extra_rows[e]),
- * row(t,j) = inv ? inv[t*k+j] : t*k+j; gates == NULL means 1 (the fan-out sum of parallel_linear_lora.py:134). */
+ * row(t,j) = inv ? inv[t*k+j] : t*k+j; gates == NULL means 1 (the fan-out sum of parallel_linear_lora.py:134);
+ * k == 0 (y may be NULL) leaves only the dense tail. */
 int moe_combine(const void* y, int64_t ldy, void* out, int64_t ldo, const void* gates, int gates_dtype,
                 const int32_t* inv, int k, int64_t ntok, int64_t ncols, int dtype, const float* extra_coef,
                 const void* extra_rows, int64_t lde, int n_extra, void* stream);

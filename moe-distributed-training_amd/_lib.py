@@ -26,6 +26,8 @@ _SIGNATURES = {
     "moe_router_topk": ("i", "ppppliiip"),
     "moe_router_forward": ("i", "plpli" + "pppp" + "lliiip"),
     "moe_router_topk_bwd": ("i", "ppppp" + "liiip"),
+    "moe_router_weight_grad_workspace_bytes": ("z", "lli"),
+    "moe_router_weight_grad": ("i", "plppllliipzp"),
     "moe_gemm_debug_plan_blocks": ("l", "lili"),
     "moe_gemm_debug_plan": ("i", "piilllii" + "pp"),
     "moe_sort_workspace_bytes": ("z", "li"),

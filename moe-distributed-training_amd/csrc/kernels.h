@@ -123,6 +123,9 @@ int moe_launch_router_topk(const float* logits, float* scores, float* topw, int3
                            int renorm, hipStream_t stream);
 int moe_launch_router_bwd(const float* dw, const float* w, const int32_t* topi, const float* scores, float* dlogits,
                           int64_t ntok, int E, int k, int renorm, hipStream_t stream);
+size_t moe_router_wgrad_ws_bytes(int64_t ntok, int64_t d, int E);
+int moe_launch_router_wgrad(const void* x, int64_t ldx, const float* dlogits, void* dwg, int64_t ldo, int64_t ntok,
+                            int64_t d, int E, int dtype, void* workspace, size_t workspace_bytes, hipStream_t stream);
 size_t moe_sort_ws_bytes(int64_t R, int E);
 int moe_launch_sort(const void* expert_idx, int in64, int64_t R, int E, int block_m, void* sorted_expert,
                     void* sorted_pos, int out64, void* counts, void* offsets, void* padded_blocks, int64_t padded_cap,

@@ -138,6 +138,17 @@ int moe_router_topk_bwd(const float* dtopw, const float* topw, const int32_t* to
     return moe_launch_router_bwd(dtopw, topw, topi, scores, dlogits, ntok, E, k, renorm, st);
 }
 
+size_t moe_router_weight_grad_workspace_bytes(int64_t ntok, int64_t d, int E) { return moe_router_wgrad_ws_bytes(ntok, d, E); }
+
+int moe_router_weight_grad(const void* x, int64_t ldx, const float* dlogits, void* dwg, int64_t ldo, int64_t ntok,
+                           int64_t d, int E, int dtype, void* workspace, size_t workspace_bytes, void* stream)
+{
+    if (ntok < 0 || d < 1 || E < 1 || !dwg || !workspace || (ntok > 0 && (!x || !dlogits))) return MOE_ERR_BAD_ARG;
+    hipStream_t st = S(stream);
+    TIMED("route.router_weight_grad");
+    return moe_launch_router_wgrad(x, ldx, dlogits, dwg, ldo, ntok, d, E, dtype, workspace, workspace_bytes, st);
+}
+
 size_t moe_sort_workspace_bytes(int64_t R, int E) { return moe_sort_ws_bytes(R, E); }
 
 int moe_sort_by_expert(const void* expert_idx, int in64, int64_t R, int E, int block_m, void* sorted_expert,
@@ -357,7 +368,7 @@ int moe_combine(const void* y, int64_t ldy, void* out, int64_t ldo, const void* 
                 const int32_t* inv, int k, int64_t ntok, int64_t ncols, int dtype, const float* extra_coef,
                 const void* extra_rows, int64_t lde, int n_extra, void* stream)
 {
-    if ((ntok > 0 && (!y || !out)) || k < 1) return MOE_ERR_BAD_ARG;
+    if (k < 0 || (ntok > 0 && (!out || (k > 0 && !y))) || (k == 0 && n_extra < 1)) return MOE_ERR_BAD_ARG;
     if (n_extra > 0 && (!extra_coef || !extra_rows)) return MOE_ERR_BAD_ARG;
     hipStream_t st = S(stream);
     TIMED("rows.combine");

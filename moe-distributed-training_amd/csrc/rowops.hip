@@ -179,6 +179,66 @@ __global__ void __launch_bounds__(ROW_THREADS) copy_rows16_kernel(const uint4* _
     for (int64_t c = threadIdx.x; c < cols16; c += ROW_THREADS) dst[r * ldd16 + c] = src[r * lds16 + c];
 }
 
+// Router weight gradient dWg[e][c] = sum_t dlogits[t][e] * x[t][c], fp32 coefficients (no rounding of dlogits), fp32
+// accumulate.  Pass 1: workgroup (chunk, column block) sums its WG_TOKENS tokens for every expert, a thread owning N
+// consecutive columns (one 16-byte load per token) and EG experts at a time; partial[chunk][e][c] fp32.  Pass 2 adds the
+// chunks in order (deterministic) and rounds once to the storage type.
+constexpr int WG_TOKENS = 64;   // tokens per partial
+constexpr int WG_EG = 8;        // experts per register block
+template <typename T>
+__global__ void __launch_bounds__(ROW_THREADS) router_wgrad_partial_kernel(const T* __restrict__ x, int64_t ldx,
+                                                                           const float* __restrict__ dl, int64_t ntok,
+                                                                           int64_t d, int E, float* __restrict__ partial,
+                                                                           int vec_ok)
+{
+    constexpr int N = Vec8<T>::N;
+    __shared__ float s_dl[WG_TOKENS * WG_EG];
+    const int64_t t0 = (int64_t)blockIdx.x * WG_TOKENS;
+    const int nt = (ntok - t0 < WG_TOKENS) ? (int)(ntok - t0) : WG_TOKENS;
+    const int64_t c0 = ((int64_t)blockIdx.y * ROW_THREADS + threadIdx.x) * N;
+    const int n = (d - c0 < N) ? (int)(d - c0) : N;
+    const bool vo = vec_ok && n == N;
+    for (int e0 = 0; e0 < E; e0 += WG_EG) {
+        const int ne = (E - e0 < WG_EG) ? E - e0 : WG_EG;
+        __syncthreads();
+        for (int i = threadIdx.x; i < WG_TOKENS * WG_EG; i += ROW_THREADS) {
+            const int tt = i / WG_EG, ee = i % WG_EG;
+            s_dl[i] = (tt < nt && ee < ne) ? dl[(t0 + tt) * E + e0 + ee] : 0.f;
+        }
+        __syncthreads();
+        if (c0 >= d) continue;
+        float acc[WG_EG][N];
+#pragma unroll
+        for (int ee = 0; ee < WG_EG; ++ee)
+#pragma unroll
+            for (int u = 0; u < N; ++u) acc[ee][u] = 0.f;
+        for (int tt = 0; tt < nt; ++tt) {
+            float v[N];
+            load_vec<T>(x + (t0 + tt) * ldx + c0, v, vo, n);
+#pragma unroll
+            for (int ee = 0; ee < WG_EG; ++ee) {
+                const float g = s_dl[tt * WG_EG + ee];
+#pragma unroll
+                for (int u = 0; u < N; ++u) acc[ee][u] = fmaf(g, v[u], acc[ee][u]);
+            }
+        }
+        for (int ee = 0; ee < ne; ++ee)
+            for (int u = 0; u < n; ++u) partial[((int64_t)blockIdx.x * E + e0 + ee) * d + c0 + u] = acc[ee][u];
+    }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(ROW_THREADS) router_wgrad_reduce_kernel(const float* __restrict__ partial, int nchunk,
+                                                                          int64_t total, int64_t d, T* __restrict__ out,
+                                                                          int64_t ldo)
+{
+    const int64_t i = (int64_t)blockIdx.x * ROW_THREADS + threadIdx.x;   // (e, c) flattened
+    if (i >= total) return;
+    float acc = 0.f;
+    for (int ch = 0; ch < nchunk; ++ch) acc += partial[(int64_t)ch * total + i];
+    Elem<T>::st(out + (i / d) * ldo + i % d, acc);
+}
+
 template <typename T> bool vec_aligned(const void* p, int64_t ld)
 {
     return ((uintptr_t)p % 16 == 0) && (ld % (16 / sizeof(T)) == 0);
@@ -253,5 +313,30 @@ int moe_launch_copy_rows_bf16(const void* src, int64_t lds_, void* dst, int64_t 
     if (cols % 8 || lds_ % 8 || ldd % 8 || ((uintptr_t)src % 16) || ((uintptr_t)dst % 16)) return MOE_ERR_UNSUPPORTED;
     hipLaunchKernelGGL(copy_rows16_kernel, dim3((unsigned)rows), dim3(ROW_THREADS), 0, stream, (const uint4*)src, lds_ / 8,
                        (uint4*)dst, ldd / 8, cols / 8);
+    return moe_launch_status();
+}
+
+size_t moe_router_wgrad_ws_bytes(int64_t ntok, int64_t d, int E)
+{
+    const int64_t nchunk = (ntok + WG_TOKENS - 1) / WG_TOKENS;
+    return (size_t)(nchunk > 0 ? nchunk : 1) * (size_t)E * (size_t)d * sizeof(float);
+}
+
+int moe_launch_router_wgrad(const void* x, int64_t ldx, const float* dlogits, void* dwg, int64_t ldo, int64_t ntok,
+                            int64_t d, int E, int dtype, void* workspace, size_t workspace_bytes, hipStream_t stream)
+{
+    if (d == 0 || E == 0) return MOE_OK;
+    if (workspace_bytes < moe_router_wgrad_ws_bytes(ntok, d, E)) return MOE_ERR_WORKSPACE;
+    const int64_t nchunk = (ntok + WG_TOKENS - 1) / WG_TOKENS;
+    const int64_t total = (int64_t)E * d;
+    MOE_DISPATCH_DTYPE(dtype, {
+        constexpr int N = Vec8<T>::N;
+        const int vo = vec_aligned<T>(x, ldx);
+        if (nchunk > 0)
+            hipLaunchKernelGGL((router_wgrad_partial_kernel<T>), dim3((unsigned)nchunk, (unsigned)((d + ROW_THREADS * N - 1) / (ROW_THREADS * N))),
+                               dim3(ROW_THREADS), 0, stream, (const T*)x, ldx, dlogits, ntok, d, E, (float*)workspace, vo);
+        hipLaunchKernelGGL((router_wgrad_reduce_kernel<T>), dim3((unsigned)((total + ROW_THREADS - 1) / ROW_THREADS)), dim3(ROW_THREADS), 0,
+                           stream, (const float*)workspace, (int)nchunk, total, d, (T*)dwg, ldo);
+    });
     return moe_launch_status();
 }

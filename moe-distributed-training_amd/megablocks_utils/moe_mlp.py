@@ -286,7 +286,7 @@ class MoELayerFn(torch.autograd.Function):
                                      offsets, k, w1.size(0))
         # fan-out sum of the k expert rows of each token plus the router's contribution dlogits @ wg, one pass
         d_x = ops.combine(dx_rows, None, k=k, extra_coef=dlogits, extra_rows=wg if wg.stride(-1) == 1 else wg.contiguous())
-        d_wg = dlogits.to(x.dtype).t() @ x if ctx.needs_input_grad[1] else None
+        d_wg = _router.router_weight_grad(x, dlogits) if ctx.needs_input_grad[1] else None
         g = grads if grads is not None else (None,) * 6
         return (d_x, d_wg) + tuple(d_w) + tuple(g) + (None, None, None)
 
@@ -306,7 +306,7 @@ def moe_layer_forward(x, wg, w1, w2, w3, top_k=2, lora: Optional[LoraViews] = No
         y = scattermoe_permute_and_compute(x, w1.reshape(E * f, d), w2.reshape(E * f, d), w3.reshape(E * f, d), f, d,
                                            top_k, sei, ssi, E, None, moe_expert_model_parallelism=False,
                                            expert_offsets=offsets, lora_views=lora, lora_alpha=lora_alpha)
-        out = _GatherCombine.apply(y, ew, inv)
+        out = _GatherCombine.apply(y, ew, inv, ssi)
         return out, ew, ei.int()
     lt = (None,) * 6 if lora is None else tuple(lora)
     return MoELayerFn.apply(x, wg, w1, w3, w2, *lt, lora_alpha, top_k, normalize)
@@ -316,21 +316,19 @@ class _GatherCombine(torch.autograd.Function):
     """out[t] = sum_j w[t,j] * y_grouped[inv[t*k+j]]  (megablocks ops.scatter, config_utils.py:251)."""
 
     @staticmethod
-    def forward(ctx, y, w, inv):
-        ctx.save_for_backward(y, w, inv)
+    def forward(ctx, y, w, inv, ssi):
+        ctx.save_for_backward(y, w, inv, ssi)
         return ops.combine(y, w, inv=inv)
 
     @staticmethod
     def backward(ctx, dout):
-        y, w, inv = ctx.saved_tensors
+        y, w, inv, ssi = ctx.saved_tensors
         dout = dout.contiguous()
         k = w.size(1)
         d_w = ops.combine_dgates(y, dout, k, w.dtype, inv=inv)
-        # dy_grouped[i] = w[pos_i] * dout[pos_i // k] with pos = inverse of inv
-        pos = torch.empty_like(inv)
-        pos[inv.long()] = torch.arange(inv.numel(), device=inv.device, dtype=inv.dtype)
-        d_y = ops.group(dout, pos, coeff=w.reshape(-1), fan_out=k)
-        return d_y, d_w, None
+        # dy_grouped[i] = w[pos_i] * dout[pos_i // k]; pos, the inverse of inv, is the sort's own sorted_scattered_idxs
+        d_y = ops.group(dout, ssi, coeff=w.reshape(-1), fan_out=k)
+        return d_y, d_w, None, None
 
 
 class ScatterMoEBlock(nn.Module):

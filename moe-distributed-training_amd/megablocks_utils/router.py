@@ -8,7 +8,7 @@ from typing import NamedTuple, Optional
 
 import torch
 
-from .._lib import lib, check, dtype_code, ptr, require_gpu, stream_ptr
+from .._lib import lib, check, dtype_code, ptr, require_gpu, stream_ptr, workspace
 from ..scattermoe_utils.kernels import ops
 
 
@@ -85,6 +85,36 @@ def router_topk_bwd(d_weights, weights, indices, scores, normalize: bool = True)
     return dl
 
 
+def router_input_grad(dlogits: torch.Tensor, weight: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """dx = dlogits @ weight from the fp32 dlogits (fp32 accumulate, one rounding to ``dtype``)."""
+    dev = require_gpu(dlogits, weight)
+    dl = dlogits.contiguous().float()
+    w = weight if weight.stride(-1) == 1 else weight.contiguous()
+    if w.dtype != dtype:
+        w = w.to(dtype)
+    T, E = dl.shape
+    d = w.size(1)
+    out = torch.empty((T, d), dtype=dtype, device=dev)
+    check(lib.moe_combine(0, 0, ptr(out), out.stride(0), 0, 0, 0, 0, T, d, dtype_code(out), ptr(dl), ptr(w), w.stride(0), E,
+                          stream_ptr(dev)), "moe_combine (router input gradient)")
+    return out
+
+
+def router_weight_grad(x2: torch.Tensor, dlogits: torch.Tensor) -> torch.Tensor:
+    """dWg = dlogits^T @ x2 from the fp32 dlogits (fp32 accumulate in a fixed order, one rounding to x2's dtype)."""
+    dev = require_gpu(x2, dlogits)
+    dl = dlogits.contiguous().float()
+    if x2.stride(-1) != 1:
+        x2 = x2.contiguous()
+    T, d = x2.shape
+    E = dl.size(1)
+    out = torch.empty((E, d), dtype=x2.dtype, device=dev)
+    ws = workspace(lib.moe_router_weight_grad_workspace_bytes(T, d, E), dev)
+    check(lib.moe_router_weight_grad(ptr(x2), x2.stride(0), ptr(dl), ptr(out), out.stride(0), T, d, E, dtype_code(x2), ptr(ws),
+                                     ws.numel(), stream_ptr(dev)), "moe_router_weight_grad")
+    return out
+
+
 class _RouterFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x2, weight, top_k, normalize):
@@ -102,9 +132,8 @@ class _RouterFn(torch.autograd.Function):
             # softmax backward for a gradient that reaches the full score matrix (e.g. an auxiliary loss)
             ds = d_scores.float()
             dl = dl + scores * (ds - (ds * scores).sum(-1, keepdim=True))
-        dlc = dl.to(x2.dtype)
-        dx = dlc @ weight if ctx.needs_input_grad[0] else None          # skinny library GEMMs (T x E x d)
-        dwg = dlc.t() @ x2 if ctx.needs_input_grad[1] else None
+        dx = router_input_grad(dl, weight, x2.dtype) if ctx.needs_input_grad[0] else None
+        dwg = router_weight_grad(x2, dl) if ctx.needs_input_grad[1] else None
         return dx, dwg, None, None
 
 
@@ -119,8 +148,8 @@ class _LogitsFn(torch.autograd.Function):
     @staticmethod
     def backward(ctx, dl):
         x2, weight = ctx.saved_tensors
-        dlc = dl.to(x2.dtype)
-        return (dlc @ weight if ctx.needs_input_grad[0] else None), (dlc.t() @ x2 if ctx.needs_input_grad[1] else None)
+        return (router_input_grad(dl, weight, x2.dtype) if ctx.needs_input_grad[0] else None,
+                router_weight_grad(x2, dl) if ctx.needs_input_grad[1] else None)
 
 
 class _TopkFn(torch.autograd.Function):

@@ -34,17 +34,23 @@ def expert_offsets_from_sorted(sorted_expert_idxs: torch.Tensor, num_experts: in
     return out
 
 
-def flatten_and_sort(expert_idxs: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+MAX_EXPERTS = 4096  # largest expert count the counting sort takes
+
+
+def flatten_and_sort(expert_idxs: torch.Tensor, num_experts: Optional[int] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """(sorted_expert_idxs, sorted_scattered_idxs): stable ascending sort of the flattened (token-major) expert
-    assignments -- the tuple megablocks_utils/config_utils.py:131-132 feeds to the kernels."""
+    assignments -- the tuple megablocks_utils/config_utils.py:131-132 feeds to the kernels.  Like the ``torch.sort`` it
+    stands in for, the sorted ids keep the input's dtype, the positions are int64, and nothing synchronises with the
+    host (so the call can be captured into a graph).  The function it replaces has no expert-count argument: without
+    ``num_experts`` the sort runs with the largest count it supports (ids must be below 4096), which costs a few
+    microseconds more than the exact count."""
     dev = require_gpu(expert_idxs)
     flat = expert_idxs.reshape(-1).contiguous()
     if flat.dtype not in (torch.int32, torch.int64):
         flat = flat.to(torch.int64)
-    R = flat.numel()
-    # the number of experts is not an argument of this function: one past the largest id (device-side max)
-    E = int(flat.max().item()) + 1 if R > 0 else 1
-    return _sort(flat, E, want_meta=False)[:2]
+    E = MAX_EXPERTS if num_experts is None else int(num_experts)
+    sei, ssi = _sort(flat, E, want_meta=False)[:2]
+    return sei, ssi if ssi.dtype == torch.int64 else ssi.long()
 
 
 def _sort(flat: torch.Tensor, E: int, want_meta: bool = True, block_m: int = BLOCK_M):

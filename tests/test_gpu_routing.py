@@ -122,6 +122,31 @@ def test_sort_bit_exact(dev, oracle, idt, R, E):
         # scattermoe's flatten_and_sort on the (T,k)-shaped tensor
         s2, p2 = ops.flatten_and_sort(t.view(-1, 1) if R % 2 else t.view(-1, 2))
         assert np.array_equal(s2.cpu().numpy(), exp["sorted_expert"]) and np.array_equal(p2.cpu().numpy(), exp["sorted_pos"])
+        assert s2.dtype == idt and p2.dtype == torch.int64          # as torch.sort: values keep the dtype, positions are int64
+        s3, p3 = ops.flatten_and_sort(t, num_experts=E)
+        assert torch.equal(s3, s2) and torch.equal(p3, p2)
+
+
+def test_flatten_and_sort_never_synchronises(dev):
+    """The drop-in flatten_and_sort (no expert-count argument, like the torch.sort it replaces) reads nothing back to the
+    host: it can be captured into a graph, and replays follow the captured buffer's new contents."""
+    _, _, ops = _mods()
+    t = torch.randint(0, 8, (4096, 2), device=dev)
+    ops.flatten_and_sort(t)                       # first call outside capture (module / attribute set-up)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        ops.flatten_and_sort(t)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        sei, ssi = ops.flatten_and_sort(t)
+    for seed in range(3):
+        t.copy_(torch.randint(0, 8, (4096, 2), generator=torch.Generator().manual_seed(seed)))
+        graph.replay()
+        torch.cuda.synchronize()
+        want_e, want_p = torch.sort(t.flatten().cpu(), stable=True)
+        assert torch.equal(sei.cpu(), want_e) and torch.equal(ssi.cpu(), want_p)
 
 
 def test_sort_is_deterministic(dev):
@@ -146,6 +171,28 @@ def test_router_backward_matches_autograd(dev, oracle):
     (w * g.to(dev)).sum().backward()
     assert torch.allclose(xg.grad.cpu(), xo.grad, atol=1e-5, rtol=1e-4)
     assert torch.allclose(wgg.grad.cpu(), wo.grad, atol=1e-5, rtol=1e-4)
+
+
+@pytest.mark.parametrize("dtype,T,d,E", [(torch.float32, 1000, 260, 8), (torch.float32, 130, 77, 19), (torch.bfloat16, 4096, 4096, 8),
+                                         (torch.bfloat16, 333, 200, 3), (torch.float16, 65, 72, 16)])
+def test_router_gradients_from_fp32_dlogits(dev, dtype, T, d, E):
+    """dWg = dlogits^T x and dx = dlogits Wg computed by the library from the fp32 dlogits (several token chunks, a
+    partial last chunk, expert counts off the register block, widths off the 16-byte vectors): fp32 inputs to 1e-5,
+    2-byte inputs to one rounding of the result (the coefficients are never rounded to the activation dtype)."""
+    _, router, _ = _mods()
+    g = torch.Generator().manual_seed(T + d)
+    x = torch.randn(T, d, generator=g).to(dtype)
+    wg = (torch.randn(E, d, generator=g) * 0.3).to(dtype)
+    dl = torch.randn(T, E, generator=g) * 0.01
+    dwg = router.router_weight_grad(x.to(dev), dl.to(dev))
+    dx = router.router_input_grad(dl.to(dev), wg.to(dev), dtype)
+    ref_w = (dl.double().t() @ x.double()).float()
+    ref_x = (dl.double() @ wg.double()).float()
+    assert dwg.dtype == dtype and dx.dtype == dtype and dwg.shape == (E, d) and dx.shape == (T, d)
+    tol = 1e-5 if dtype == torch.float32 else (2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -10)
+    assert float((dwg.float().cpu() - ref_w).abs().max() / ref_w.abs().max()) < tol
+    assert float((dx.float().cpu() - ref_x).abs().max() / ref_x.abs().max()) < tol
+    assert torch.equal(dwg, router.router_weight_grad(x.to(dev), dl.to(dev)))      # fixed summation order
 
 
 @pytest.mark.parametrize("case", ["bias", "p2", "bias_p2_k1", "no_norm", "jitter", "uniform"])
