@@ -244,14 +244,17 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
     // A image: row r at r*128 B, logical 16-byte chunk c of that row at slot c ^ ((r >> 1) & 7): two rows span the
     // 64 LDS banks, so 16 consecutive rows of one chunk column hit 16 different bank groups.
     // Wave w issues load instructions j = 0..3; instruction (j, w) fills rows [(j*8 + w)*8, +8).
+    // Grouped rows are addressed from the tile's first row (the descriptor is re-based there, so the 32-bit offsets
+    // only span one tile whatever the number of rows); gathered rows from the start of X.
+    const int64_t a_row_base = p.x_grouped ? row0 : 0;
     uint32_t a_off[LPT];   // byte offsets into X[0] / X[1] (the same for both K segments)
 #pragma unroll
     for (int j = 0; j < LPT; ++j) {
         const int r = (j * NWAVES + wave) * 8 + (lane >> 3);
         const int c = (lane & 7) ^ ((r >> 1) & 7);
-        a_off[j] = (uint32_t)((s_inrow[r] * p.ldx + c * 8) * 2);
+        a_off[j] = (uint32_t)(((s_inrow[r] - a_row_base) * p.ldx + c * 8) * 2);
     }
-    const i32x4_t a_buf0 = make_buffer(p.X[0]), a_buf1 = make_buffer(p.X[1] ? p.X[1] : p.X[0]);
+    const i32x4_t a_buf0 = make_buffer(p.X[0] + a_row_base * p.ldx), a_buf1 = make_buffer((p.X[1] ? p.X[1] : p.X[0]) + a_row_base * p.ldx);
     // B: offsets within this expert's matrix.  For the SwiGLU pair image rows [0,128) come from W[0] and [128,256)
     // from W[1], which are whole load instructions (the first and second half of a wave's LPT); otherwise W[0] / W[1]
     // are the two K segments.
@@ -674,19 +677,31 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
     // get an offset past the descriptor's range, which the hardware drops, so the loop has no branches.
     auto stage_flush = [&](int sw, uint16_t* Y, int64_t ld, bool scattered, int64_t ncol0) {
         __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's staging writes have landed
-        const __amdgpu_buffer_rsrc_t ybuf = __builtin_amdgcn_make_buffer_rsrc(Y, 0, (int)0x80000000u, 0x00020000);
+        // grouped rows: the descriptor starts at the tile's first row, so offsets stay within one tile
+        const __amdgpu_buffer_rsrc_t ybuf = __builtin_amdgcn_make_buffer_rsrc(scattered ? Y : Y + row0 * ld, 0, (int)0x80000000u, 0x00020000);
         const int lpr = sw / 8, rows_per_it = 64 / lpr, iters = WTM / rows_per_it;
         const int slot = lane % lpr;
         const uint32_t ld2 = (uint32_t)ld * 2;
+        if (scattered && p.y_wide) {
+            // scattered rows of an output beyond the 2 GiB a descriptor offset spans: 64-bit addresses, a branch per lane
+            for (int it = 0; it < iters; ++it) {
+                const int m = it * rows_per_it + lane / lpr;
+                const u32x4_t v = *(const u32x4_t*)(stg + m * (sw * 2) + slot * 16);
+                const int rl = wm * WTM + m;
+                const int64_t n = ncol0 + swz(sw, m, slot) * 8;
+                if (rl < nrows && n < p.N) *(u32x4_t*)(Y + s_outrow[rl] * ld + n) = v;
+            }
+        } else {
 #pragma unroll 8
-        for (int it = 0; it < iters; ++it) {
-            const int m = it * rows_per_it + lane / lpr;
-            const u32x4_t v = *(const u32x4_t*)(stg + m * (sw * 2) + slot * 16);
-            const int rl = wm * WTM + m;
-            const int64_t n = ncol0 + swz(sw, m, slot) * 8;
-            const uint32_t orow = scattered ? (uint32_t)s_outrow[rl] : (uint32_t)(row0 + rl);
-            const uint32_t off = (rl < nrows && n < p.N) ? orow * ld2 + (uint32_t)n * 2 : 0xFFFFFFF0u;
-            __builtin_amdgcn_raw_buffer_store_b128(v, ybuf, off, 0, 0);
+            for (int it = 0; it < iters; ++it) {
+                const int m = it * rows_per_it + lane / lpr;
+                const u32x4_t v = *(const u32x4_t*)(stg + m * (sw * 2) + slot * 16);
+                const int rl = wm * WTM + m;
+                const int64_t n = ncol0 + swz(sw, m, slot) * 8;
+                const uint32_t orow = scattered ? (uint32_t)s_outrow[rl] : (uint32_t)rl;
+                const uint32_t off = (rl < nrows && n < p.N) ? orow * ld2 + (uint32_t)n * 2 : 0xFFFFFFF0u;
+                __builtin_amdgcn_raw_buffer_store_b128(v, ybuf, off, 0, 0);
+            }
         }
         __builtin_amdgcn_s_waitcnt(0xC07F);  // reads done before the slice is reused
     };
@@ -737,10 +752,11 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
         // dh (scaled by the row's routing weight) is staged as bf16 -- the precision a stored dh would have -- and
         // then revisited row segment by row segment: 8 lanes cover 128 bytes of a row, so the matching gate / up
         // values are fetched, and dgate / dup written, with full-width coalesced accesses.
-        const __amdgpu_buffer_rsrc_t gbuf = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p.H1), 0, (int)0x80000000u, 0x00020000);
-        const __amdgpu_buffer_rsrc_t ubuf = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p.H3), 0, (int)0x80000000u, 0x00020000);
-        const __amdgpu_buffer_rsrc_t dgbuf = __builtin_amdgcn_make_buffer_rsrc(p.Y[0], 0, (int)0x80000000u, 0x00020000);
-        const __amdgpu_buffer_rsrc_t dubuf = __builtin_amdgcn_make_buffer_rsrc(p.Y[1], 0, (int)0x80000000u, 0x00020000);
+        // (all four are grouped rows: descriptors start at the tile's first row)
+        const __amdgpu_buffer_rsrc_t gbuf = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p.H1) + row0 * p.ldh, 0, (int)0x80000000u, 0x00020000);
+        const __amdgpu_buffer_rsrc_t ubuf = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p.H3) + row0 * p.ldh, 0, (int)0x80000000u, 0x00020000);
+        const __amdgpu_buffer_rsrc_t dgbuf = __builtin_amdgcn_make_buffer_rsrc(p.Y[0] + row0 * p.ldy, 0, (int)0x80000000u, 0x00020000);
+        const __amdgpu_buffer_rsrc_t dubuf = __builtin_amdgcn_make_buffer_rsrc(p.Y[1] + row0 * p.ldy, 0, (int)0x80000000u, 0x00020000);
         // gate / up are read once and dgate / dup written once per launch: the non-temporal hint keeps them from
         // displacing operand tiles in L2 (measured: this kernel 2 % faster; on the plain output stores it is slower)
         constexpr int STREAMING = 2;
@@ -756,7 +772,7 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
             const int rl = wm * WTM + m;
             const int64_t n = n0 + wn * WTN + swz(WTN, m, slot) * 8;
             const bool valid = rl < nrows && n < p.N;
-            const uint32_t row = (uint32_t)(row0 + rl);
+            const uint32_t row = (uint32_t)rl;
             hoff = valid ? row * ldh2 + (uint32_t)n * 2 : 0xFFFFFFF0u;   // out of range: reads zeros, writes nothing
             yoff = valid ? row * ldy2 + (uint32_t)n * 2 : 0xFFFFFFF0u;
         };
@@ -833,6 +849,7 @@ template <bool NN, int EPI> int launch_variant(const MoeGemmParams& p, int64_t R
     const int ntiles_n = (EPI == MOE_EPI_SWIGLU) ? (int)((p.N + BN / 2 - 1) / (BN / 2)) : (int)((p.N + BN - 1) / BN);
     MoeGemmParams q = p;
     q.num_cus = moe_num_cus();
+    q.y_wide = (!p.y_grouped && (R * p.ldy + p.N) * 2 >= ((int64_t)1 << 31)) ? 1 : 0;
     q.max_split = moe_gemm_max_split(EPI == MOE_EPI_SWIGLU);
     if (q.max_split > 1) {
         if (!p.sk_partials || !p.sk_counters) return MOE_ERR_WORKSPACE;
@@ -887,13 +904,17 @@ bool moe_gemm_mfma_supported(const MoeGemmParams& p, int64_t R)
     for (int i = 0; i < MOE_MAX_SLABS; ++i)
         if (!al16(p.Q[i]) || !al16(p.LB[i])) return false;
     if (p.nseg < 1 || p.nseg > 2 || p.nslab < 0 || p.nslab > MOE_MAX_SLABS || (p.slab_mode == 1 && p.nslab % 2 != 0)) return false;
-    // operand tiles are addressed with 32-bit byte offsets from the start of X and of one expert's matrix
-    const int64_t x_rows = p.x_grouped ? R : (R + (p.fan_out > 0 ? p.fan_out : 1) - 1) / (p.fan_out > 0 ? p.fan_out : 1);
+    // 32-bit byte offsets: gathered A rows from the start of X (grouped ones from the tile's first row), weights from
+    // the start of one expert's matrix, grouped outputs and the saved gate / up from the tile's first row; scattered
+    // output rows from the start of Y while Y spans less than 2 GiB, 64-bit addresses beyond (y_wide, set at launch)
+    (void)R;
+    const int fo = p.fan_out > 0 ? p.fan_out : 1;
+    const int64_t x_rows = p.x_grouped ? BM : (R + fo - 1) / fo;
     const int64_t limit = (int64_t)1 << 32;
     if ((x_rows * p.ldx + p.K) * 2 >= limit) return false;
     if (((p.nn ? p.K : p.N) * p.ldw + (p.nn ? p.N : p.K)) * 2 >= limit) return false;
-    if ((R * p.ldy + p.N) * 2 >= limit / 2) return false;   // output tiles: buffer stores with a 2 GiB range
-    if (p.epi == MOE_EPI_SWIGLU_BWD && (R * p.ldh + p.N) * 2 >= limit / 2) return false;   // gate / up tiles likewise
+    if ((BM * p.ldy + p.N) * 2 >= limit / 2) return false;
+    if (p.epi == MOE_EPI_SWIGLU_BWD && (BM * p.ldh + p.N) * 2 >= limit / 2) return false;
     return true;
 }
 

@@ -94,11 +94,11 @@ __global__ void __launch_bounds__(NTHREADS) grouped_xty_mfma_kernel(const MoeXty
         const int j = is_b ? idx : idx - LPT;
         const int left = nrows - kt * BR;
         const uint32_t row_bytes = is_b ? b_row_bytes : a_row_bytes;
-        const uint64_t base = (is_b ? b_base : a_base) + (uint64_t)(uint32_t)(kt * BR) * row_bytes;
+        const uint64_t base = (is_b ? b_base : a_base) + (uint64_t)(kt * BR) * row_bytes;   // 64-bit: a group may span more than 4 GiB
         i32x4_t rsrc;
         rsrc.x = __builtin_amdgcn_readfirstlane((int)(uint32_t)base);
         rsrc.y = __builtin_amdgcn_readfirstlane((int)(uint32_t)(base >> 32));
-        rsrc.z = __builtin_amdgcn_readfirstlane((int)(left > 0 ? (uint32_t)left * row_bytes : 0u));
+        rsrc.z = __builtin_amdgcn_readfirstlane((int)(left > 0 ? (uint32_t)(left < BR ? left : BR) * row_bytes : 0u));   // a step reads BR rows at most
         rsrc.w = 0x00020000;
         load_to_lds_16(rsrc, is_b ? b_off[j] : a_off[j], smem_u + (kt & 1) * STAGE_BYTES + (is_b ? OP_BYTES : 0) + j * (NWAVES * 1024));
     };
@@ -239,9 +239,11 @@ bool moe_xty_mfma_supported(const MoeXtyParams& p, int64_t R)
     auto al16 = [](const void* q) { return q != nullptr && ((uintptr_t)q % 16) == 0; };
     if (p.K <= 0 || p.N <= 0 || p.K % 8 != 0 || p.N % 8 != 0 || p.ldx % 8 != 0 || p.ldy % 8 != 0 || p.ldw % 8 != 0 || p.swe % 8 != 0) return false;
     if (!al16(p.X) || !al16(p.DY) || !al16(p.DW)) return false;
-    // operand tiles are addressed with 32-bit byte offsets inside one group's rows, output tiles inside one expert's matrix
+    // operand tiles are addressed with 32-bit byte offsets from the first row of one contraction step (descriptors are
+    // re-based per step), output tiles inside one expert's matrix: no limit on the number of rows
+    (void)R;
     const int64_t limit = (int64_t)1 << 31;
-    if ((R * p.ldx + p.K) * 2 >= limit || (R * p.ldy + p.N) * 2 >= limit) return false;
+    if ((BR * p.ldx + p.K) * 2 >= limit || (BR * p.ldy + p.N) * 2 >= limit) return false;
     if ((p.K * p.ldw + p.N) * 2 >= limit) return false;
     return true;
 }

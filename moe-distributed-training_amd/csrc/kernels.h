@@ -40,6 +40,7 @@ struct MoeGemmParams {
     int x_grouped;
     int y_grouped;
     int epi;
+    int y_wide;             // scattered output rows need 64-bit addresses (Y spans 2 GiB or more), set by the launcher
     int max_split;          // K parts a tile of the last round may be cut into (1, 2 or 4), set by the launcher
     int num_cus;            // compute units the tile plan fills (a multiple of 8), set by the launcher
     float* sk_partials;     // K-split exchange area, see moe_gemm_sk_bytes / moe_gemm_sk_attach

@@ -427,6 +427,14 @@ static bool mlp_shapes_ok(int64_t d, int64_t f, int64_t ldx, int rank, const voi
     return d % 64 == 0 && f % 64 == 0 && ldx % 8 == 0 && rank <= 32 && aligned16(a) && aligned16(b) && aligned16(c) &&
            aligned16(x);
 }
+// What the grouped GEMM's 32-bit offsets allow, checked before anything is enqueued: gathered rows are addressed from
+// the start of their matrix (below 4 GiB), one expert's weight matrix likewise, one 256-row tile of the (R, f)
+// intermediates below 2 GiB.  The number of rows itself is not limited.
+static bool mlp_sizes_ok(int64_t gathered_rows, int64_t ld_gathered, int64_t d, int64_t f)
+{
+    const int64_t g4 = (int64_t)1 << 32;
+    return (gathered_rows * ld_gathered + d) * 2 < g4 && (f * d + d) * 2 < g4 && (256 * f + f) * 2 < g4 / 2 && (256 * (d + 64) + d) * 2 < g4 / 2;
+}
 
 int moe_mlp_fwd(const void* x, int64_t ldx, const void* w1, const void* w3, const void* w2, const void* const* lora,
                 const int64_t* ls, int rank, float scaling, void* gate, void* up, void* h, void* y, int64_t ldy,
@@ -437,6 +445,7 @@ int moe_mlp_fwd(const void* x, int64_t ldx, const void* w1, const void* w3, cons
     const bool has_lora = lora && lora[0];
     if (has_lora && (!ls || !saved || rank < 1)) return MOE_ERR_BAD_ARG;
     if (!mlp_shapes_ok(d, f, ldx, has_lora ? rank : 0, w1, w3, w2, x)) return MOE_ERR_UNSUPPORTED;
+    if (!mlp_sizes_ok(R / fan_out, bad_pitch(ldx) ? d + 64 : ldx, d, f)) return MOE_ERR_UNSUPPORTED;
     if (R == 0) return MOE_OK;
     hipStream_t st = S(stream);
     uint8_t* sv = (uint8_t*)saved;
@@ -546,6 +555,7 @@ int moe_mlp_bwd(const void* dy, int64_t lddy, int dy_grouped, int dy_fan_out, co
     if (!mlp_shapes_ok(d, f, ldx, has_lora ? rank : 0, w1, w3, w2, x) || lddy % 8 != 0 || !aligned16(dy))
         return MOE_ERR_UNSUPPORTED;
     if (dy_fan_out < 1 || fan_out < 1) return MOE_ERR_BAD_ARG;
+    if (!mlp_sizes_ok(dy_grouped ? 256 : R / dy_fan_out, bad_pitch(lddy) ? d + 64 : lddy, d, f)) return MOE_ERR_UNSUPPORTED;
     hipStream_t st = S(stream);
     const size_t qb = q_bytes(R);
     const int64_t ldt = pad_rows(R);

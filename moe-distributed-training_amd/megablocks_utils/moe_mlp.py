@@ -68,6 +68,10 @@ def _fast_path_ok(x, w1, w2, w3, lora: Optional[LoraViews]) -> bool:
         return False
     if lora is not None and lora.a1.size(2) > 32:   # the fused launches take an adapter as one or two 16-wide rank chunks
         return False
+    # gathered activation rows and one expert's matrix are addressed with 32-bit byte offsets (the same check the library
+    # makes before it enqueues anything); the number of rows is otherwise not limited
+    if (x.size(0) * (d + 64) + d) * 2 >= 1 << 32 or (f * d + d) * 2 >= 1 << 32:
+        return False
     return True
 
 

@@ -58,3 +58,22 @@ def test_cpu_tensors_fail_loudly():
         moe.flatten_and_sort(torch.tensor([1, 0, 1]))
     with pytest.raises(RuntimeError, match="GPU only"):
         moe.forward_router(torch.randn(4, 8), torch.randn(2, 8), 1)
+
+
+def test_size_limits_are_checked_before_anything_is_enqueued():
+    """The fused entry points address gathered activation rows and one expert's matrix with 32-bit byte offsets; sizes
+    beyond that are refused on the host with MOE_ERR_UNSUPPORTED (status codes only: nothing is dereferenced), while the
+    number of rows alone never is (grouped tiles are addressed from their own first row)."""
+    from moe_distributed_training_amd._lib import lib
+    one = 16   # non-null, 16-byte aligned stand-ins: rejected before any use
+
+    def fwd(R, d, f, fan_out):
+        return lib.moe_mlp_fwd(one, d, one, one, one, None, None, 0, 0.0, one, one, one, one, d, one, 0, one, 0, 8,
+                               R, d, f, fan_out, 0, None, None, 0, None)
+    # a gathered x of 4 GiB or more: T * (d + 64) * 2 bytes
+    assert fwd(2 * 600000, 4096, 14336, 2) == -2
+    # one expert's matrix of 4 GiB or more
+    assert fwd(8192, 65536, 32768, 2) == -2
+    # many rows alone are fine: the call gets as far as the workspace check (status -3), i.e. past the size checks
+    assert fwd(2 * 200000, 4096, 14336, 2) == -3
+    assert lib.moe_mlp_workspace_bytes(400000, 8, 4096, 14336, 16) > 0

@@ -509,6 +509,50 @@ def test_skewed_full_size_properties(dev, oracle):
                 check_expert_grads(g1[n][j][e:e + 1], loe[n][j].grad[e:e + 1], f"{nm} {n} expert {e} ({tok.numel()} rows)")
 
 
+@pytest.mark.slow
+def test_layer_with_intermediates_above_2GiB(dev, oracle):
+    """T=40960 tokens (R=81920 rows) at the Mixtral shape: gate, up, h, dgate and dup are 2.35 GB each, beyond what a
+    32-bit byte offset from the tensor's start reaches in the SwiGLU epilogues.  Tokens are independent, so out and dX of
+    slices of the batch (the first rows, the last rows, the rows around the 2 GiB mark of the grouped order is not
+    addressable by token -- slices spread over the batch) equal the fp32 oracle run on those slices alone."""
+    import moe_distributed_training_amd as moe
+    T, d, f, E, k, r, alpha = 40960, 4096, 14336, 8, 2, 16, 32.0
+    g = torch.Generator(device=dev).manual_seed(8)
+    rn = lambda *s, std=1.0: (torch.randn(*s, generator=g, device=dev) * std).bfloat16()
+    x, wg = rn(T, d), rn(E, d, std=0.02)
+    w1, w2, w3 = rn(E, f, d, std=0.02), rn(E, f, d, std=0.02), rn(E, f, d, std=0.02)
+    lora = {"w1": (rn(E, d, r, std=0.02), rn(E, r, f, std=0.02)), "w3": (rn(E, d, r, std=0.02), rn(E, r, f, std=0.02)),
+            "w2": (rn(E, f, r, std=0.02), rn(E, r, d, std=0.02))}
+    dout = rn(T, d)
+    lt, views = _views({n: (a.cpu(), b.cpu()) for n, (a, b) in lora.items()}, dev)
+    xg = x.clone().requires_grad_(True)
+    out, ew, ei = moe.moe_layer_forward(xg, wg, w1, w2, w3, k, views, alpha)
+    out.backward(dout)
+    torch.cuda.synchronize()
+    assert T * k * f * 2 > (1 << 31)
+    torch.set_num_threads(16)
+    W = [t.float().cpu() for t in (wg, w1, w2, w3)]
+    lo = {n: (a.float().cpu(), b.float().cpu()) for n, (a, b) in lora.items()}
+    for sl in (slice(0, 192), slice(T // 2 - 96, T // 2 + 96), slice(T - 192, T)):
+        xo = x[sl].float().cpu().requires_grad_(True)
+        ref, aux = oracle.moe_block(xo, W[0], W[1], W[2], W[3], k, lo, alpha)
+        ref.backward(dout[sl].float().cpu())
+        assert torch.equal(ei[sl].cpu().long(), aux["indices"])
+        assert rel(out[sl], ref) < 1e-2 and rel(xg.grad[sl], xo.grad) < 1e-2, sl
+    # adapter gradients of the last expert -- its rows sit at the end of the grouped order, past the 2 GiB mark of every
+    # (R, f) tensor -- against the oracle run on the tokens routed to it (one assignment each, the layer's own weight)
+    e = E - 1
+    ewc, eic = ew.detach().float().cpu(), ei.cpu().long()
+    tok, slot = torch.where(eic == e)
+    loe = {n: (a.float().cpu().requires_grad_(True), b.float().cpu().requires_grad_(True)) for n, (a, b) in lora.items()}
+    refe, _ = oracle.moe_block(x[tok.to(dev)].float().cpu(), None, W[1], W[2], W[3], 1, loe, alpha,
+                               routing=(ewc[tok, slot][:, None], torch.full((tok.numel(), 1), e)))
+    refe.backward(dout[tok.to(dev)].float().cpu())
+    for n in ("w1", "w3", "w2"):
+        for j, nm in ((0, "dA"), (1, "dB")):
+            check_expert_grads(lt[n][j].grad[e:e + 1], loe[n][j].grad[e:e + 1], f"{nm} {n} expert {e} ({tok.numel()} rows)")
+
+
 def test_step_captures_into_a_graph_and_replays_bit_identically(dev):
     """The library enqueues kernels only (no host synchronisation, no memset nodes, no allocation of its own), so a
     whole forward+backward step can be captured into a HIP graph.  Every replay -- with eager work and synchronisations

@@ -110,6 +110,42 @@ def test_k_split_exchange_is_stable_over_many_launches(dev, oracle, T, E, k, K, 
             assert int(bad.item()) == 0, f"a launch among {i + 2 - check_every}..{i + 1} differs from the first"
 
 
+@pytest.mark.slow
+@pytest.mark.parametrize("case", ["grouped_out_above_2GiB", "scattered_out_above_2GiB", "grouped_in_above_4GiB"])
+def test_scatter2scatter_beyond_32_bit_spans(dev, case):
+    """Tensors larger than a 32-bit byte offset reaches: a grouped output above 2 GiB (tiles addressed from their own
+    first row), a scattered output above 2 GiB (64-bit row addresses) and a grouped input above 4 GiB.  Rows from the
+    first tile, the last tile and around the 2 / 4 GiB marks against per-row fp32 products."""
+    ops = _ops()
+    g = torch.Generator(device=dev).manual_seed(31)
+    E = 4
+    if case == "grouped_in_above_4GiB":
+        R, K, N = 140000, 16384, 64
+    else:
+        R, K, N = 70000, 64, 16384
+    counts = [R // 2 - 777, 0, R // 4 + 500, R - (R // 2 - 777) - (R // 4 + 500)]
+    eo = torch.tensor(counts).cumsum(0)
+    sei = torch.repeat_interleave(torch.arange(E), torch.tensor(counts)).to(dev)
+    scattered = case == "scattered_out_above_2GiB"
+    ssi = (torch.randperm(R, generator=torch.Generator().manual_seed(32)) if scattered else torch.arange(R)).to(dev)
+    X = torch.randn(R, K, generator=g, device=dev).bfloat16()
+    W = (torch.randn(E, K, N, generator=g, device=dev) * 0.05).bfloat16()
+    assert max(X.numel(), R * N) * 2 > (1 << 31)
+    y = ops.scatter2scatter(X, W, sei, ssi, 1, None, True, not scattered)
+    torch.cuda.synchronize()
+    mark = (1 << 31) // (2 * N) if case != "grouped_in_above_4GiB" else (1 << 32) // (2 * K)
+    rows = sorted(set(list(range(0, 300)) + list(range(R - 300, R)) + list(range(mark - 300, mark + 300)) +
+                      [int(v) for v in eo.tolist() if 0 < v < R] + [int(v) - 1 for v in eo.tolist() if v > 0]))
+    m = torch.tensor(rows, device=dev)
+    e_of = sei[m]
+    ref = torch.bmm(X[m].float().unsqueeze(1), W.float()[e_of]).squeeze(1)
+    got = y[ssi[m] if scattered else m].float()
+    assert float((got - ref).abs().max() / ref.abs().max()) < 1e-2
+    if scattered:   # every output row was written exactly once: a permutation of the grouped result
+        yg = ops.scatter2scatter(X, W, sei, ssi, 1, None, True, True)
+        assert torch.equal(y[ssi], yg)
+
+
 def test_scatter2scatter_out_argument_and_empty(dev, oracle):
     ops = _ops()
     torch.manual_seed(2)
