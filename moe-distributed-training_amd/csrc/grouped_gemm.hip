@@ -57,6 +57,11 @@ constexpr int LDS_BYTES = NSTAGE_A * A_STAGE_BYTES + NSTAGE_B * B_STAGE_BYTES;  
 // main loop's first tile that stage is still empty, and after the loop the epilogue staging only needs the first 128 KiB.
 constexpr int TABLE_OFF = B_REGION + 2 * B_STAGE_BYTES;
 static_assert(TABLE_OFF >= NWAVES * (BM / 2) * (BN / (NWAVES / 2)) * 2, "epilogue staging must not reach the tables");
+// SwiGLU-backward epilogue with fused row contractions: images of three [BM][16] bf16 operands sit behind the row tables
+constexpr int RC_MATS = 3;
+constexpr int RC_IMG_OFF = TABLE_OFF + 2 * BM * 8 + 64;
+constexpr int RC_IMG_BYTES = BM * 16 * 2;                       // 8 KiB per operand
+static_assert(RC_IMG_OFF + RC_MATS * RC_IMG_BYTES <= LDS_BYTES, "row-contraction images fit behind the tables");
 constexpr int NXCD = 8;
 constexpr int INTERLEAVE_MIN_ROUNDS = 8;    // launches with at least this many rounds of tiles deal them to the XCDs in chunks
 
@@ -95,6 +100,7 @@ struct WorkItem {
     int part, nparts;          // K part of a split tile (0 of 1: whole tile)
     int split_item;            // exchange slot of this part (the slots of a tile are consecutive, in part order)
     int split_tile;            // counter of the split tile
+    int mtile;                 // number of the row tile among all row tiles (experts in order, BM rows each)
 };
 
 __device__ __forceinline__ WorkItem decode_work_item(const void* offsets, int off64, int E, int ntiles_n, int ktiles,
@@ -165,9 +171,10 @@ __device__ __forceinline__ WorkItem decode_work_item(const void* offsets, int of
         w.nt = __builtin_amdgcn_readfirstlane(nt);
         w.row0 = uniform_i64(row0);
         w.row1 = uniform_i64(row1);
+        w.mtile = __builtin_amdgcn_readfirstlane((int)(before + mt));
         w.valid = true;
     } else {
-        int64_t start = 0, id = t;
+        int64_t start = 0, id = t, mtiles_before = 0;
         for (int e = 0; e < E; ++e) {
             const int64_t end = load_idx(offsets, e, off64);
             const int64_t mte = (end - start + BM - 1) / BM;
@@ -176,12 +183,14 @@ __device__ __forceinline__ WorkItem decode_work_item(const void* offsets, int of
                 w.expert = e;
                 w.nt = (int)(id / mte);
                 const int64_t mt = id % mte;
+                w.mtile = (int)(mtiles_before + mt);
                 w.row0 = start + mt * BM;
                 w.row1 = (w.row0 + BM < end) ? w.row0 + BM : end;
                 w.valid = true;
                 break;
             }
             id -= te;
+            mtiles_before += mte;
             start = end;
         }
     }
@@ -784,6 +793,21 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
         };
 #pragma unroll
         for (int it = 0; it < PD; ++it) fetch(it, it);
+        // ---- fused row contractions (adapter gradients that sum over the rows of dgate, dup and h): for the tile's rows,
+        //   RCP[0][mtile][n][r] = sum_m dgate[m][n] RC[0][m][r],  RCP[1] likewise with dup and RC[1],
+        //   RCP[2][mtile][n][r] = sum_m h[m][n] RC[2][m][r],  h = silu(gate) * up recomputed here (bit-identical to the
+        //   forward's h: same operands, same order),
+        // so that none of the three (R, N) tensors is read from memory again for them.  A per-expert reduction over
+        // the row tiles (in order) finishes the sums.  The operands RC (bf16 [R][16]) are brought into LDS once per tile.
+        const bool rc = p.nrc > 0;
+        uint8_t* rc_img = smem + RC_IMG_OFF;
+        u32x4_t rc_in[RC_MATS];
+        if (rc) {
+            const int r_ = tid >> 1;                                   // tile row of this thread's 16 bytes
+            const int64_t m_ = row0 + (r_ < nrows ? r_ : nrows - 1);   // rows past the group re-read its last row (they meet zeros)
+#pragma unroll
+            for (int mat = 0; mat < RC_MATS; ++mat) rc_in[mat] = *(const u32x4_t*)(p.RC[mat] + m_ * 16 + (tid & 1) * 8);
+        }
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
@@ -791,33 +815,131 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
                 const float s_ = rs[mb];
                 stage_put(WTN, mb * 16 + mrow, nb * 16 + nq, pack4(acc[mb][nb][0] * s_, acc[mb][nb][1] * s_, acc[mb][nb][2] * s_, acc[mb][nb][3] * s_));
             }
+        if (rc) {
+            static_assert(NTHREADS * 16 == RC_IMG_BYTES, "one 16-byte piece of every operand image per thread");
+#pragma unroll
+            for (int mat = 0; mat < RC_MATS; ++mat) *(u32x4_t*)(rc_img + mat * RC_IMG_BYTES + tid * 16) = rc_in[mat];
+            __syncthreads();   // the images are complete (and, for this wave, its dh staging)
+        }
         __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's staging writes have landed
+        // transposing reads (see the N-contiguous weight fragments): lane 16g + i fetches 4 columns at row 8g + (i >> 2)
+        // and 4 rows further down, and receives rows 8g .. 8g+7 of column i -- a 16x16x32 operand whose contraction
+        // index is the row.  Offsets within a block of 32 rows of this wave's staging slice / of an operand image.
+        const int tg = lane >> 4, ti = lane & 15;
+        const int trow = 8 * tg + (ti >> 2);
+        constexpr int IBLK = WTN / 16;   // 16-column blocks of the wave's sub-tile
+        f32x4_t rcd[RC_MATS][IBLK];
 #pragma unroll
-        for (int it = 0; it < NIT; ++it) {
-            const int m = it * ROWS_PER_IT + lane / LPR;
-            const u32x4_t dh8 = *(const u32x4_t*)(stg + m * (WTN * 2) + slot * 16);
-            uint32_t hoff, yoff;
-            seg_addr(it, hoff, yoff);
-            const u32x4_t gg = g8[it % PD], uu = u8[it % PD];
-            u32x4_t og8, ou8;
+        for (int mat = 0; mat < RC_MATS; ++mat)
 #pragma unroll
-            for (int w2 = 0; w2 < 4; ++w2) {
-                float og[2], ou[2];
+            for (int ib = 0; ib < IBLK; ++ib) rcd[mat][ib] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+        auto tr_read = [&](const uint8_t* p0, const uint8_t* p1) {
+            s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)LDS_PTR(p0));
+            s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)LDS_PTR(p1));
+            union { struct { s16x4_t a, b; } s; bf16x8_t v; } u;
+            u.s.a = lo; u.s.b = hi;
+            return u.v;
+        };
+        constexpr int BLK_ITS = 32 / ROWS_PER_IT;   // row segments per block of 32 rows
+        static_assert(NIT % BLK_ITS == 0 && PD <= BLK_ITS, "whole blocks of 32 rows");
 #pragma unroll
-                for (int t = 0; t < 2; ++t) {
-                    const float g = bf16_bits_to_f32((uint16_t)(gg[w2] >> (t * 16)));
-                    const float u = bf16_bits_to_f32((uint16_t)(uu[w2] >> (t * 16)));
-                    const float dh = bf16_bits_to_f32((uint16_t)(dh8[w2] >> (t * 16)));
-                    const float sg = sigmoid_f(g);
-                    og[t] = dh * u * sg * (1.f + g * (1.f - sg));
-                    ou[t] = dh * g * sg;
+        for (int blk = 0; blk < NIT / BLK_ITS; ++blk) {
+            u32x4_t og8[BLK_ITS], ou8[BLK_ITS], hh8[BLK_ITS];
+#pragma unroll
+            for (int q = 0; q < BLK_ITS; ++q) {
+                const int it = blk * BLK_ITS + q;
+                const int m = it * ROWS_PER_IT + lane / LPR;
+                const u32x4_t dh8 = *(const u32x4_t*)(stg + m * (WTN * 2) + slot * 16);
+                uint32_t hoff, yoff;
+                seg_addr(it, hoff, yoff);
+                const u32x4_t gg = g8[it % PD], uu = u8[it % PD];
+#pragma unroll
+                for (int w2 = 0; w2 < 4; ++w2) {
+                    float og[2], ou[2], hh[2];
+#pragma unroll
+                    for (int t = 0; t < 2; ++t) {
+                        const float g = bf16_bits_to_f32((uint16_t)(gg[w2] >> (t * 16)));
+                        const float u = bf16_bits_to_f32((uint16_t)(uu[w2] >> (t * 16)));
+                        const float dh = bf16_bits_to_f32((uint16_t)(dh8[w2] >> (t * 16)));
+                        const float sg = sigmoid_f(g);
+                        og[t] = dh * u * sg * (1.f + g * (1.f - sg));
+                        ou[t] = dh * g * sg;
+                        hh[t] = g * sg * u;
+                    }
+                    og8[q][w2] = pack_bf16x2(og[0], og[1]);
+                    ou8[q][w2] = pack_bf16x2(ou[0], ou[1]);
+                    hh8[q][w2] = pack_bf16x2(hh[0], hh[1]);
+                    // Rows past the group must enter the contractions as exact zeros.  Their gate / up read as zeros, but
+                    // their dh need not be finite: the accumulators of row blocks without real rows can hold anything (an
+                    // MFMA that the compiler left under an execution mask instead of a branch runs all the same -- the
+                    // matrix cores ignore the mask -- on fragments of rows that were never loaded), and 0 * inf is not 0.
+                    if (rc && wm * WTM + m >= nrows) og8[q][w2] = ou8[q][w2] = 0u;
                 }
-                og8[w2] = pack_bf16x2(og[0], og[1]);
-                ou8[w2] = pack_bf16x2(ou[0], ou[1]);
+                if (it + PD < NIT) fetch(it + PD, it % PD);
+                __builtin_amdgcn_raw_buffer_store_b128(og8[q], dgbuf, yoff, 0, STREAMING);
+                __builtin_amdgcn_raw_buffer_store_b128(ou8[q], dubuf, yoff, 0, STREAMING);
             }
-            if (it + PD < NIT) fetch(it + PD, it % PD);
-            __builtin_amdgcn_raw_buffer_store_b128(og8, dgbuf, yoff, 0, STREAMING);
-            __builtin_amdgcn_raw_buffer_store_b128(ou8, dubuf, yoff, 0, STREAMING);
+            if (rc) {
+                // the block's 32 rows of this wave's slice have been consumed: dgate, dup and h take their place in turn
+                // (same swizzled positions), each read back transposed and contracted with its operand image.  LDS serves
+                // a wave's requests in order, so the three write / read rounds are queued back to back without waiting
+                // for one another; the MFMAs follow when the fragments arrive.
+                const uint8_t* blk_img = stg + blk * 32 * (WTN * 2);
+                bf16x8_t pf[RC_MATS], vf[RC_MATS][IBLK];
+#pragma unroll
+                for (int mat = 0; mat < RC_MATS; ++mat) {
+#pragma unroll
+                    for (int q = 0; q < BLK_ITS; ++q) {
+                        const int m = (blk * BLK_ITS + q) * ROWS_PER_IT + lane / LPR;
+                        *(u32x4_t*)(stg + m * (WTN * 2) + slot * 16) = mat == 0 ? og8[q] : (mat == 1 ? ou8[q] : hh8[q]);
+                    }
+                    asm volatile("" ::: "memory");   // the reads below follow the writes above in program order
+                    const uint8_t* pim = rc_img + mat * RC_IMG_BYTES + (wm * WTM + blk * 32 + trow) * 32 + (ti & 3) * 8;
+                    pf[mat] = tr_read(pim, pim + 4 * 32);
+#pragma unroll
+                    for (int ib = 0; ib < IBLK; ++ib) {
+                        const int c = 2 * ib + ((ti & 3) >> 1), half = ti & 1;
+                        const int r0_ = blk * 32 + trow, r1_ = r0_ + 4;   // rows within the slice (their swizzle term is (row >> 1) & 7)
+                        const uint8_t* a0 = blk_img + trow * (WTN * 2) + ((c ^ ((r0_ >> 1) & 7)) << 4) + half * 8;
+                        const uint8_t* a1 = blk_img + (trow + 4) * (WTN * 2) + ((c ^ ((r1_ >> 1) & 7)) << 4) + half * 8;
+                        vf[mat][ib] = tr_read(a0, a1);
+                    }
+                    asm volatile("" ::: "memory");   // ... and the next operand's writes follow these reads
+                }
+#pragma unroll
+                for (int mat = 0; mat < RC_MATS; ++mat)
+#pragma unroll
+                    for (int ib = 0; ib < IBLK; ++ib)
+                        rcd[mat][ib] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[mat][ib], pf[mat], rcd[mat][ib], 0, 0, 0);
+            }
+        }
+        if (rc) {
+            // rcd[mat][ib][reg] = element (column ib*16 + 4*(lane/16) + reg, rank column lane%16) summed over this wave's
+            // 128 rows: the lower row of waves hands its sums to the upper one (through its staging slice), which adds
+            // them in a fixed order and stores the tile's partial
+            __builtin_amdgcn_s_waitcnt(0xC07F);
+            // (a wave of the lower row writes into its own slice, which it has finished with; the upper one reads it there)
+            float* xch = (float*)(smem + ((wave % WAVES_N) + WAVES_N) * (WTM * WTN * 2));
+            if (wm == 1) {
+#pragma unroll
+                for (int mat = 0; mat < RC_MATS; ++mat)
+#pragma unroll
+                    for (int ib = 0; ib < IBLK; ++ib)
+                        *(f32x4_t*)(xch + ((mat * IBLK + ib) * 64 + lane) * 4) = rcd[mat][ib];
+            }
+            __syncthreads();
+            if (wm == 0) {
+#pragma unroll
+                for (int mat = 0; mat < RC_MATS; ++mat)
+#pragma unroll
+                    for (int ib = 0; ib < IBLK; ++ib) {
+                        const f32x4_t o = *(const f32x4_t*)(xch + ((mat * IBLK + ib) * 64 + lane) * 4);
+                        float* dst = p.RCP[mat] + ((int64_t)item.mtile * p.N + n0 + wn * WTN + ib * 16 + 4 * tg) * 16 + ti;
+#pragma unroll
+                        for (int reg = 0; reg < 4; ++reg)
+                            if (n0 + wn * WTN + ib * 16 + 4 * tg + reg < p.N) dst[reg * 16] = rcd[mat][ib][reg] + o[reg];
+                    }
+            }
         }
     }
 }
@@ -887,13 +1009,13 @@ size_t moe_gemm_sk_bytes(int64_t R, int E, int64_t N)
 {
     const int64_t tiles = (R / BM + E) * ((N + BN - 1) / BN);
     const int64_t slots = 4 * tiles < moe_num_cus() ? 4 * tiles : moe_num_cus();
-    return (size_t)moe_num_cus() * sizeof(int) + 256 + (size_t)slots * BM * BN * sizeof(float);
+    return (size_t)moe_gemm_num_counters() * sizeof(int) + 256 + (size_t)slots * BM * BN * sizeof(float);
 }
 
 void moe_gemm_sk_attach(MoeGemmParams& p, void* ws, int64_t, int, int64_t)
 {
     p.sk_counters = (int*)ws;
-    p.sk_partials = (float*)((uint8_t*)ws + (((size_t)moe_num_cus() * sizeof(int) + 255) & ~(size_t)255));
+    p.sk_partials = (float*)((uint8_t*)ws + (((size_t)moe_gemm_num_counters() * sizeof(int) + 255) & ~(size_t)255));
 }
 
 bool moe_gemm_mfma_supported(const MoeGemmParams& p, int64_t R)
@@ -927,3 +1049,4 @@ int moe_launch_gemm_mfma(const MoeGemmParams& p, int64_t R, hipStream_t stream)
     if (p.epi == MOE_EPI_SWIGLU_BWD) return p.nn ? launch_variant<true, MOE_EPI_SWIGLU_BWD>(p, R, stream) : launch_variant<false, MOE_EPI_SWIGLU_BWD>(p, R, stream);
     return MOE_ERR_BAD_ARG;
 }
+

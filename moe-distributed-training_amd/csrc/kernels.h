@@ -28,6 +28,12 @@ struct MoeGemmParams {
     const uint16_t* H1;     // saved gate / up for MOE_EPI_SWIGLU_BWD
     const uint16_t* H3;
     int64_t ldh;
+    // MOE_EPI_SWIGLU_BWD only: fused row contractions (nrc = 0 or 3).  RC[i]: bf16 [R][16] operands in grouped order;
+    // RCP[i]: fp32 partials [row tile][N][16], row tiles of 256 rows per expert in order (the layout the fixed-order
+    // reduction of the adapter gradients sums): RCP[0] = dgate^T RC[0], RCP[1] = dup^T RC[1], RCP[2] = h^T RC[2]
+    const uint16_t* RC[3];
+    float* RCP[3];
+    int nrc;
     const float* row_scale; // optional per sorted position factor applied to the accumulator (STORE, SWIGLU_BWD)
     const void* pos;        // sorted_scattered_idxs
     int pos64;
@@ -98,11 +104,17 @@ int moe_launch_rows_lora(const void* X, int64_t ldx, const void* At, void* Q, vo
                          int pos64, const void* offsets, int off64, int E, int64_t R, int64_t K, int fan_out,
                          int x_grouped, float scaling, const float* qt_row_scale, hipStream_t stream);
 // two products over the same rows in one launch (X2 == nullptr: only the first)
+// q_scaled (optional): a third output of the first product, [R][16] like Q but multiplied by qt_row_scale like Qt
 int moe_launch_rows_lora2(const void* X, const void* X2, int64_t ldx, const void* At, const void* At2, void* Q, void* Q2,
                           void* Qt, void* Qt2, int64_t ldqt, const void* pos, int pos64, const void* offsets, int off64,
                           int E, int64_t R, int64_t K, int fan_out, int x_grouped, float scaling,
-                          const float* qt_row_scale, hipStream_t stream);
+                          const float* qt_row_scale, hipStream_t stream, void* q_scaled = nullptr);
 size_t moe_xtp_workspace_bytes(int64_t R, int E, int64_t K);
+// the reduction half of moe_launch_xtp2 alone, for partials [row tile of 256][K][16] that another kernel produced
+// (partial2 == nullptr: only the first)
+int moe_launch_xtp_reduce2(const float* partial, const float* partial2, void* out, void* out2, const int64_t* so,
+                           const int64_t* so2, int rank, int rank2, const void* offsets, int off64, int E, int64_t K,
+                           float scale, hipStream_t stream);
 // two reductions over the same rows in one launch pair (X2 == nullptr: only the first); so / so2: output strides
 // {expert, k, r}; rank / rank2: columns each writes; needs twice moe_xtp_workspace_bytes when X2 is given
 int moe_launch_xtp2(const void* X, const void* X2, int64_t ldx, const void* pos, int pos64, int fan_out, const void* Pt,

@@ -89,7 +89,7 @@ static_assert(RL_KSTEPS == RL_WAVES, "one K step per wave and stage");
 // lanes touch different rows, which the memory pipeline handles one lane at a time.  All global loads of the loop are
 // inline assembly with explicit s_waitcnt: compiler-managed loads would wait for the prefetches queued behind them.
 // one or two jobs per launch (blockIdx.y): same rows, shapes and scaling, different operand / output pointers
-struct RowsLoraJob { const uint16_t* X; const uint16_t* Af; uint16_t* Q; uint16_t* Qt; };
+struct RowsLoraJob { const uint16_t* X; const uint16_t* Af; uint16_t* Q; uint16_t* Qt; uint16_t* Qs; };   // Qs: optional row-major copy scaled like Qt
 // ROWS = 32 rows per workgroup, or 16 when a launch of 32-row tiles would leave most compute units with a single
 // workgroup (and so with too few loads in flight)
 template <int ROWS>
@@ -187,7 +187,9 @@ __global__ void __launch_bounds__(RL_THREADS) rows_lora_kernel(const RowsLoraJob
             for (int w = 0; w < RL_WAVES; ++w) v += red[w][row][col];
             v *= scaling;
             Q[mo * 16 + col] = f32_to_bf16_bits(v);
-            if (Qt) Qt[(int64_t)col * ldqt + mo] = f32_to_bf16_bits(qt_row_scale ? v * qt_row_scale[mo] : v);
+            const float vs = qt_row_scale ? v * qt_row_scale[mo] : v;
+            if (Qt) Qt[(int64_t)col * ldqt + mo] = f32_to_bf16_bits(vs);
+            if (job.Qs) job.Qs[mo * 16 + col] = f32_to_bf16_bits(vs);
         }
     }
 }
@@ -355,7 +357,7 @@ int moe_launch_pack_lora_batch(const MoePackBatch& jobs, hipStream_t stream)
 int moe_launch_rows_lora2(const void* X, const void* X2, int64_t ldx, const void* At, const void* At2, void* Q, void* Q2,
                           void* Qt, void* Qt2, int64_t ldqt, const void* pos, int pos64, const void* offsets, int off64,
                           int E, int64_t R, int64_t K, int fan_out, int x_grouped, float scaling,
-                          const float* qt_row_scale, hipStream_t stream)
+                          const float* qt_row_scale, hipStream_t stream, void* q_scaled)
 {
     if (R == 0) return MOE_OK;
     const bool two = X2 != nullptr;
@@ -369,8 +371,8 @@ int moe_launch_rows_lora2(const void* X, const void* X2, int64_t ldx, const void
             return MOE_ERR_LAUNCH;
         attr_set = true;
     }
-    const RowsLoraJob j0 = {(const uint16_t*)X, (const uint16_t*)At, (uint16_t*)Q, (uint16_t*)Qt};
-    const RowsLoraJob j1 = {(const uint16_t*)X2, (const uint16_t*)At2, (uint16_t*)Q2, (uint16_t*)Qt2};
+    const RowsLoraJob j0 = {(const uint16_t*)X, (const uint16_t*)At, (uint16_t*)Q, (uint16_t*)Qt, (uint16_t*)q_scaled};
+    const RowsLoraJob j1 = {(const uint16_t*)X2, (const uint16_t*)At2, (uint16_t*)Q2, (uint16_t*)Qt2, nullptr};
     // 32-row tiles halve the adapter traffic, but two workgroups fit a compute unit: use them when the launch has
     // about that many, otherwise 16-row tiles (three fit)
     static std::atomic<int> cus{0};
@@ -428,6 +430,21 @@ int moe_launch_xtp2(const void* X, const void* X2, int64_t ldx, const void* pos,
     dim3 rgrid((unsigned)((K * 16 + 255) / 256), (unsigned)E, two ? 2u : 1u);
     hipLaunchKernelGGL(xtp_reduce_kernel, rgrid, dim3(256), 0, stream, (const float*)workspace, pstride, j0, j1, offsets,
                        off64, E, K, scale);
+    return moe_launch_status();
+}
+
+int moe_launch_xtp_reduce2(const float* partial, const float* partial2, void* out, void* out2, const int64_t* so,
+                           const int64_t* so2, int rank, int rank2, const void* offsets, int off64, int E, int64_t K,
+                           float scale, hipStream_t stream)
+{
+    if (E == 0 || K == 0) return MOE_OK;
+    const bool two = partial2 != nullptr;
+    if (rank < 1 || rank > 16 || (two && (rank2 < 1 || rank2 > 16))) return MOE_ERR_UNSUPPORTED;
+    const XtpJob j0 = {nullptr, nullptr, (uint16_t*)out, so[0], so[1], so[2], rank};
+    const XtpJob j1 = two ? XtpJob{nullptr, nullptr, (uint16_t*)out2, so2[0], so2[1], so2[2], rank2} : j0;
+    dim3 rgrid((unsigned)((K * 16 + 255) / 256), (unsigned)E, two ? 2u : 1u);
+    hipLaunchKernelGGL(xtp_reduce_kernel, rgrid, dim3(256), 0, stream, partial, two ? (int64_t)(partial2 - partial) : 0, j0, j1,
+                       offsets, off64, E, K, scale);
     return moe_launch_status();
 }
 

@@ -5,6 +5,7 @@
 #include "kernels.h"
 #include <mutex>
 #include <string.h>
+#include <stdlib.h>
 #include <vector>
 
 namespace {
@@ -416,7 +417,7 @@ size_t moe_mlp_workspace_bytes(int64_t R, int E, int64_t d, int64_t f, int rank)
     if (rank <= 0) return n;
     const int64_t mx = d > f ? d : f;
     const size_t C = (size_t)(rank + 15) / 16;   // 16-wide chunks per adapter
-    return n + C * (3 * pack_bytes(E, d) + 3 * pack_bytes(E, f) + 6 * q_bytes(R)) + al(2 * moe_xtp_workspace_bytes(R, E, mx));
+    return n + C * (3 * pack_bytes(E, d) + 3 * pack_bytes(E, f) + 7 * q_bytes(R)) + al(3 * moe_xtp_workspace_bytes(R, E, mx));
 }
 
 size_t moe_mlp_saved_bytes(int64_t R, int rank) { return rank > 0 ? (size_t)((rank + 15) / 16) * 6 * q_bytes(R) : 256; }
@@ -568,7 +569,11 @@ int moe_mlp_bwd(const void* dy, int64_t lddy, int dy_grouped, int dy_fan_out, co
     auto pqp = [&](int which, int c) { return pq + ((size_t)c * 6 + which) * qb; };   // which: 0 P2, 1 P1, 2 P3, 3 P2t, 4 P1t, 5 P3t
     auto svp = [&](int which, int c) { return sv + ((size_t)c * 6 + which) * qb; };   // which: 0 Q1, 1 Q3, 2 Q2, 3 Qt1, 4 Qt3, 5 Qt2
     void* xw = nullptr;
+    void* p2s = nullptr;
     size_t xb = 0;
+    // a rank of at most 16 (one chunk): the adapter gradients that sum over the rows of dgate, dup and h are produced by
+    // the dh GEMM's epilogue as per-row-tile partials; two chunks take the separate passes over those tensors
+    const bool fuse_rc = has_lora && rank <= 16 && getenv("MOE_NO_FUSE_RC") == nullptr;
     if (!workspace || workspace_bytes < moe_mlp_workspace_bytes(R, E, d, f, has_lora ? rank : 0)) return MOE_ERR_WORKSPACE;
     Bump ws(workspace, workspace_bytes);
     void* skws = ws.take(sk_bytes_mlp(R, E, d, f));
@@ -584,8 +589,9 @@ int moe_mlp_bwd(const void* dy, int64_t lddy, int dy_grouped, int dy_fan_out, co
     }
     if (has_lora) {
         pq = (uint8_t*)ws.take((size_t)C * 6 * qb);
+        if (fuse_rc) p2s = ws.take(qb);   // P2 times the row scale, row-major (the fused contraction's operand)
         const int64_t mx = d > f ? d : f;
-        xb = 2 * moe_xtp_workspace_bytes(R, E, mx);   // paired reductions keep two sets of partials
+        xb = 3 * moe_xtp_workspace_bytes(R, E, mx);   // paired reductions keep two sets of partials, the fused ones of the dh GEMM three
         xw = ws.take(xb);
         TIMED("bwd.pack_lora");
         MoePackBatch pb = {};
@@ -618,7 +624,7 @@ int moe_mlp_bwd(const void* dy, int64_t lddy, int dy_grouped, int dy_fan_out, co
         TIMED("bwd.rows_lora_dy");
         TRY(moe_launch_rows_lora2(dy, C > 1 ? dy : nullptr, lddy, bt2[0], bt2[1], pqp(0, 0), C > 1 ? pqp(0, 1) : nullptr, pqp(3, 0),
                                   C > 1 ? pqp(3, 1) : nullptr, ldt, pos, pos64, offsets, off64, E, R, d, dy_fan_out, dy_grouped, scaling,
-                                  row_scale, st));
+                                  row_scale, st, p2s));
     }
     {
         MoeGemmParams p = {};
@@ -633,6 +639,12 @@ int moe_mlp_bwd(const void* dy, int64_t lddy, int dy_grouped, int dy_fan_out, co
         p.pos = pos; p.pos64 = pos64; p.offsets = offsets; p.off64 = off64;
         p.E = E; p.K = d; p.N = f; p.fan_out = dy_fan_out; p.x_grouped = dy_grouped; p.y_grouped = 1;
         p.epi = MOE_EPI_SWIGLU_BWD;
+        if (fuse_rc) {   // dB1 = Q1^T dgate, dB3 = Q3^T dup, dA2 = h^T (row_scale P2) as per-row-tile partials from the epilogue
+            const size_t one = moe_xtp_workspace_bytes(R, E, f);
+            p.RC[0] = (const uint16_t*)svp(0, 0); p.RC[1] = (const uint16_t*)svp(1, 0); p.RC[2] = (const uint16_t*)p2s;
+            for (int i = 0; i < 3; ++i) p.RCP[i] = (float*)((uint8_t*)xw + i * one);
+            p.nrc = 3;
+        }
         moe_gemm_sk_attach(p, skws, R, E, f);
         p.counters_clean = counters_clean;
         if (moe_gemm_max_split(p.epi == MOE_EPI_SWIGLU) > 1) counters_clean = true;   // zeroed by that launch if they were not, and left zero
@@ -641,10 +653,17 @@ int moe_mlp_bwd(const void* dy, int64_t lddy, int dy_grouped, int dy_fan_out, co
     }
     if (has_lora) {
         // dA2[e][k=f][r] = sum_m h[m][k] * (row_scale[m] P2[m][r]);  dB2[e][r][n=d] = sum_m (row_scale[m] Q2[m][r]) dy[m][n]
+        const int64_t sb1[3] = {gs[3], gs[5], gs[4]}, sb3[3] = {gs[9], gs[11], gs[10]};
         { TIMED("bwd.xtp_w2");
         const int64_t sa2[3] = {gs[12], gs[13], gs[14]}, sb2[3] = {gs[15], gs[17], gs[16]};
         uint16_t* dA2 = (uint16_t*)lg[4];
         uint16_t* dB2 = (uint16_t*)lg[5];
+        if (fuse_rc) {   // the sums over each row tile came out of the dh GEMM's epilogue: add the tiles per expert
+            const size_t one = moe_xtp_workspace_bytes(R, E, f);
+            const float* part = (const float*)xw;
+            TRY(moe_launch_xtp_reduce2(part, part + one / sizeof(float), lg[1], lg[3], sb1, sb3, rank, rank, offsets, off64, E, f, 1.f, st));
+            TRY(moe_launch_xtp_reduce2(part + 2 * (one / sizeof(float)), nullptr, dA2, nullptr, sa2, nullptr, rank, 0, offsets, off64, E, f, 1.f, st));
+        } else
         TRY(moe_launch_xtp2(h, C > 1 ? h : nullptr, f, nullptr, 0, 1, pqp(3, 0), C > 1 ? pqp(3, 1) : nullptr, ldt, nullptr, dA2,
                             C > 1 ? dA2 + 16 * gs[14] : nullptr, sa2, sa2, rank < 16 ? rank : 16, C > 1 ? rank - 16 : 0, offsets, off64, E, R, f,
                             1.f, xw, xb, st));
@@ -686,6 +705,7 @@ int moe_mlp_bwd(const void* dy, int64_t lddy, int dy_grouped, int dy_fan_out, co
             const int rk = (rank - 16 * c < 16) ? rank - 16 * c : 16;
             TRY(moe_launch_xtp2(x, x, ldx, pos, pos64, fan_out, pqp(4, c), pqp(5, c), ldt, nullptr, (uint16_t*)lg[0] + 16 * c * gs[2],
                                 (uint16_t*)lg[2] + 16 * c * gs[8], sa1, sa3, rk, rk, offsets, off64, E, R, d, 1.f, xw, xb, st));
+            if (!fuse_rc)
             TRY(moe_launch_xtp2(dgate, dup, f, nullptr, 0, 1, svp(3, c), svp(4, c), ldt, nullptr, (uint16_t*)lg[1] + 16 * c * gs[4],
                                 (uint16_t*)lg[3] + 16 * c * gs[10], sb1, sb3, rk, rk, offsets, off64, E, R, f, 1.f, xw, xb, st));
         }
