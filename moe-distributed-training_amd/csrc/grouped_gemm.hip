@@ -793,16 +793,20 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
         };
 #pragma unroll
         for (int it = 0; it < PD; ++it) fetch(it, it);
-        // ---- fused row contractions (adapter gradients that sum over the rows of dgate, dup and h): for the tile's rows,
-        //   RCP[0][mtile][n][r] = sum_m dgate[m][n] RC[0][m][r],  RCP[1] likewise with dup and RC[1],
-        //   RCP[2][mtile][n][r] = sum_m h[m][n] RC[2][m][r],  h = silu(gate) * up recomputed here (bit-identical to the
-        //   forward's h: same operands, same order),
-        // so that none of the three (R, N) tensors is read from memory again for them.  A per-expert reduction over
-        // the row tiles (in order) finishes the sums.  The operands RC (bf16 [R][16]) are brought into LDS once per tile.
-        const bool rc = p.nrc > 0;
+        // ---- fused low-rank products (EPI = MOE_EPI_SWIGLU_BWD_FUSED): while dgate, dup and h = silu(gate) * up (recomputed
+        // here, bit-identical to the forward's h: same operands, same order) pass through LDS, the tile also produces
+        //   row contractions (adapter gradients that sum over the tile's rows m):
+        //     RCP[0][mtile][n][r] = sum_m dgate[m][n] RC[0][m][r],  RCP[1] likewise with dup and RC[1],  RCP[2] with h and RC[2]
+        //   column contractions (the low-rank interims of the next GEMM, sums over the tile's columns n):
+        //     CCP[0][nt][m][r] = sum_n dgate[m][n] CB[0][e][n][r],  CCP[1] likewise with dup and CB[1]
+        // so that none of the three (R, N) tensors is read from memory again for them.  Small reduction kernels add the
+        // row tiles per expert / the column tiles (in order), scale and round.  RC: bf16 [R][16] in grouped order, brought
+        // into LDS once per tile; CB: adapter factor in MFMA fragment order (lane i + 16 g of fragment kb holds
+        // factor[32 kb + 8 g .. + 7][i]).
+        constexpr bool FUSED = EPI == MOE_EPI_SWIGLU_BWD_FUSED;
         uint8_t* rc_img = smem + RC_IMG_OFF;
         u32x4_t rc_in[RC_MATS];
-        if (rc) {
+        if (FUSED) {
             const int r_ = tid >> 1;                                   // tile row of this thread's 16 bytes
             const int64_t m_ = row0 + (r_ < nrows ? r_ : nrows - 1);   // rows past the group re-read its last row (they meet zeros)
 #pragma unroll
@@ -815,7 +819,7 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
                 const float s_ = rs[mb];
                 stage_put(WTN, mb * 16 + mrow, nb * 16 + nq, pack4(acc[mb][nb][0] * s_, acc[mb][nb][1] * s_, acc[mb][nb][2] * s_, acc[mb][nb][3] * s_));
             }
-        if (rc) {
+        if (FUSED) {
             static_assert(NTHREADS * 16 == RC_IMG_BYTES, "one 16-byte piece of every operand image per thread");
 #pragma unroll
             for (int mat = 0; mat < RC_MATS; ++mat) *(u32x4_t*)(rc_img + mat * RC_IMG_BYTES + tid * 16) = rc_in[mat];
@@ -828,11 +832,24 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
         const int tg = lane >> 4, ti = lane & 15;
         const int trow = 8 * tg + (ti >> 2);
         constexpr int IBLK = WTN / 16;   // 16-column blocks of the wave's sub-tile
-        f32x4_t rcd[RC_MATS][IBLK];
+        constexpr int CC_MATS = 2, CC_KS = WTN / 32;
+        f32x4_t rcd[RC_MATS][IBLK];      // row contractions, accumulated over the wave's 128 rows
+        bf16x8_t cbf[CC_MATS][CC_KS];    // this wave's fragments of the two adapter factors
+        if (FUSED) {
 #pragma unroll
-        for (int mat = 0; mat < RC_MATS; ++mat)
+            for (int mat = 0; mat < RC_MATS; ++mat)
 #pragma unroll
-            for (int ib = 0; ib < IBLK; ++ib) rcd[mat][ib] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+                for (int ib = 0; ib < IBLK; ++ib) rcd[mat][ib] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int mat = 0; mat < CC_MATS; ++mat)
+#pragma unroll
+                for (int ks = 0; ks < CC_KS; ++ks) {
+                    const int64_t ncol = n0 + wn * WTN + ks * 32;
+                    bf16x8_t v = {};
+                    if (ncol < p.N) v = *(const bf16x8_t*)(p.CB[mat] + ((int64_t)expert * p.N + ncol) * 16 + lane * 8);
+                    cbf[mat][ks] = v;
+                }
+        }
         auto tr_read = [&](const uint8_t* p0, const uint8_t* p1) {
             s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)LDS_PTR(p0));
             s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)LDS_PTR(p1));
@@ -840,6 +857,7 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
             u.s.a = lo; u.s.b = hi;
             return u.v;
         };
+        const int cc_frag_off = (lane & 15) * (WTN * 2);   // + (chunk ^ swizzle) * 16 per read
         constexpr int BLK_ITS = 32 / ROWS_PER_IT;   // row segments per block of 32 rows
         static_assert(NIT % BLK_ITS == 0 && PD <= BLK_ITS, "whole blocks of 32 rows");
 #pragma unroll
@@ -868,26 +886,31 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
                     }
                     og8[q][w2] = pack_bf16x2(og[0], og[1]);
                     ou8[q][w2] = pack_bf16x2(ou[0], ou[1]);
-                    hh8[q][w2] = pack_bf16x2(hh[0], hh[1]);
+                    if (FUSED) hh8[q][w2] = pack_bf16x2(hh[0], hh[1]);
                     // Rows past the group must enter the contractions as exact zeros.  Their gate / up read as zeros, but
                     // their dh need not be finite: the accumulators of row blocks without real rows can hold anything (an
                     // MFMA that the compiler left under an execution mask instead of a branch runs all the same -- the
                     // matrix cores ignore the mask -- on fragments of rows that were never loaded), and 0 * inf is not 0.
-                    if (rc && wm * WTM + m >= nrows) og8[q][w2] = ou8[q][w2] = 0u;
+                    if (FUSED && wm * WTM + m >= nrows) og8[q][w2] = ou8[q][w2] = 0u;
                 }
                 if (it + PD < NIT) fetch(it + PD, it % PD);
                 __builtin_amdgcn_raw_buffer_store_b128(og8[q], dgbuf, yoff, 0, STREAMING);
                 __builtin_amdgcn_raw_buffer_store_b128(ou8[q], dubuf, yoff, 0, STREAMING);
             }
-            if (rc) {
-                // the block's 32 rows of this wave's slice have been consumed: dgate, dup and h take their place in turn
-                // (same swizzled positions), each read back transposed and contracted with its operand image.  LDS serves
-                // a wave's requests in order, so the three write / read rounds are queued back to back without waiting
-                // for one another; the MFMAs follow when the fragments arrive.
-                const uint8_t* blk_img = stg + blk * 32 * (WTN * 2);
-                bf16x8_t pf[RC_MATS], vf[RC_MATS][IBLK];
+            if (FUSED) {
+                // The block's 32 rows of this wave's slice have been consumed: dgate, dup and h take their place in turn
+                // (same swizzled positions); each is read back transposed for its row contraction and, dgate and dup,
+                // row-major for the column contractions.  LDS serves a wave's requests in order, so the next operand's
+                // writes and reads are queued behind the current one's reads before its MFMAs start.
+                uint8_t* blk_img = stg + blk * 32 * (WTN * 2);
+                bf16x8_t pf[2], vf[2][IBLK], cf[2][2][CC_KS];   // two generations of fragments
+                f32x4_t ccd[CC_MATS][2];                          // column contractions of the block's two 16-row blocks
 #pragma unroll
-                for (int mat = 0; mat < RC_MATS; ++mat) {
+                for (int mat = 0; mat < CC_MATS; ++mat)
+#pragma unroll
+                    for (int rb = 0; rb < 2; ++rb) ccd[mat][rb] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+                auto queue = [&](int mat) {
+                    const int gen = mat & 1;
 #pragma unroll
                     for (int q = 0; q < BLK_ITS; ++q) {
                         const int m = (blk * BLK_ITS + q) * ROWS_PER_IT + lane / LPR;
@@ -895,30 +918,81 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
                     }
                     asm volatile("" ::: "memory");   // the reads below follow the writes above in program order
                     const uint8_t* pim = rc_img + mat * RC_IMG_BYTES + (wm * WTM + blk * 32 + trow) * 32 + (ti & 3) * 8;
-                    pf[mat] = tr_read(pim, pim + 4 * 32);
+                    pf[gen] = tr_read(pim, pim + 4 * 32);
 #pragma unroll
                     for (int ib = 0; ib < IBLK; ++ib) {
                         const int c = 2 * ib + ((ti & 3) >> 1), half = ti & 1;
                         const int r0_ = blk * 32 + trow, r1_ = r0_ + 4;   // rows within the slice (their swizzle term is (row >> 1) & 7)
                         const uint8_t* a0 = blk_img + trow * (WTN * 2) + ((c ^ ((r0_ >> 1) & 7)) << 4) + half * 8;
                         const uint8_t* a1 = blk_img + (trow + 4) * (WTN * 2) + ((c ^ ((r1_ >> 1) & 7)) << 4) + half * 8;
-                        vf[mat][ib] = tr_read(a0, a1);
+                        vf[gen][ib] = tr_read(a0, a1);
+                    }
+                    if (mat < CC_MATS) {
+#pragma unroll
+                        for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+                            for (int ks = 0; ks < CC_KS; ++ks)
+                                cf[gen][rb][ks] = *(const bf16x8_t*)(blk_img + rb * 16 * (WTN * 2) + cc_frag_off + (((ks * 4 + (lane >> 4)) ^ ((lane >> 1) & 7)) << 4));
                     }
                     asm volatile("" ::: "memory");   // ... and the next operand's writes follow these reads
-                }
-#pragma unroll
-                for (int mat = 0; mat < RC_MATS; ++mat)
+                };
+                auto consume = [&](int mat) {
+                    const int gen = mat & 1;
 #pragma unroll
                     for (int ib = 0; ib < IBLK; ++ib)
-                        rcd[mat][ib] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[mat][ib], pf[mat], rcd[mat][ib], 0, 0, 0);
+                        rcd[mat][ib] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[gen][ib], pf[gen], rcd[mat][ib], 0, 0, 0);
+                    if (mat < CC_MATS) {
+#pragma unroll
+                        for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+                            for (int ks = 0; ks < CC_KS; ++ks)
+                                ccd[mat][rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cf[gen][rb][ks], cbf[mat][ks], ccd[mat][rb], 0, 0, 0);
+                    }
+                };
+                queue(0);
+                queue(1);
+                consume(0);
+                queue(2);
+                consume(1);
+                consume(2);
+                // the block's column contractions are complete (they only sum over this wave's 64 columns): they take the
+                // block's place in the slice -- 4 KiB, [product][16-row block][lane] -- until the waves exchange them below
+#pragma unroll
+                for (int mat = 0; mat < CC_MATS; ++mat)
+#pragma unroll
+                    for (int rb = 0; rb < 2; ++rb)
+                        *(f32x4_t*)(blk_img + ((mat * 2 + rb) * 64 + lane) * 16) = ccd[mat][rb];
             }
         }
-        if (rc) {
-            // rcd[mat][ib][reg] = element (column ib*16 + 4*(lane/16) + reg, rank column lane%16) summed over this wave's
-            // 128 rows: the lower row of waves hands its sums to the upper one (through its staging slice), which adds
-            // them in a fixed order and stores the tile's partial
+        if (FUSED) {
+            // column contractions: element (row = 16-row block * 16 + 4 * (lane / 16) + reg, rank column lane % 16) summed
+            // over one wave's 64 columns sits in that wave's slice; wave (wm, wn) adds the four column waves' sums (in wave
+            // order) for the 32-row block wn of its row half and stores them
             __builtin_amdgcn_s_waitcnt(0xC07F);
-            // (a wave of the lower row writes into its own slice, which it has finished with; the upper one reads it there)
+            __syncthreads();
+#pragma unroll
+            for (int mat = 0; mat < CC_MATS; ++mat)
+#pragma unroll
+                for (int rb = 0; rb < 2; ++rb) {
+                    f32x4_t sum = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int w2 = 0; w2 < WAVES_N; ++w2) {
+                        const uint8_t* src = smem + (wm * WAVES_N + w2) * (WTM * WTN * 2) + wn * 32 * (WTN * 2);
+                        const f32x4_t v = *(const f32x4_t*)(src + ((mat * 2 + rb) * 64 + lane) * 16);
+#pragma unroll
+                        for (int reg = 0; reg < 4; ++reg) sum[reg] += v[reg];
+                    }
+                    const int rl0 = wm * WTM + wn * 32 + rb * 16 + 4 * tg;
+                    float* dst = p.CCP[mat] + ((int64_t)nt * p.cc_rows + row0 + rl0) * 16 + ti;
+#pragma unroll
+                    for (int reg = 0; reg < 4; ++reg)
+                        if (rl0 + reg < nrows) dst[reg * 16] = sum[reg];
+                }
+            __builtin_amdgcn_s_waitcnt(0xC07F);
+            __syncthreads();   // the slices are free again for the exchange below
+            // row contractions: rcd[mat][ib][reg] = element (column ib*16 + 4*(lane/16) + reg, rank column lane%16) summed
+            // over this wave's 128 rows: the lower row of waves parks its sums in its own slices, the upper one adds them
+            // to its own (a fixed order) and stores the tile's partial
             float* xch = (float*)(smem + ((wave % WAVES_N) + WAVES_N) * (WTM * WTN * 2));
             if (wm == 1) {
 #pragma unroll
@@ -1036,7 +1110,7 @@ bool moe_gemm_mfma_supported(const MoeGemmParams& p, int64_t R)
     if ((x_rows * p.ldx + p.K) * 2 >= limit) return false;
     if (((p.nn ? p.K : p.N) * p.ldw + (p.nn ? p.N : p.K)) * 2 >= limit) return false;
     if ((BM * p.ldy + p.N) * 2 >= limit / 2) return false;
-    if (p.epi == MOE_EPI_SWIGLU_BWD && (BM * p.ldh + p.N) * 2 >= limit / 2) return false;
+    if ((p.epi == MOE_EPI_SWIGLU_BWD || p.epi == MOE_EPI_SWIGLU_BWD_FUSED) && (BM * p.ldh + p.N) * 2 >= limit / 2) return false;
     return true;
 }
 
@@ -1047,6 +1121,11 @@ int moe_launch_gemm_mfma(const MoeGemmParams& p, int64_t R, hipStream_t stream)
     if (p.epi == MOE_EPI_STORE) return p.nn ? launch_variant<true, MOE_EPI_STORE>(p, R, stream) : launch_variant<false, MOE_EPI_STORE>(p, R, stream);
     if (p.epi == MOE_EPI_SWIGLU) return p.nn ? MOE_ERR_UNSUPPORTED : launch_variant<false, MOE_EPI_SWIGLU>(p, R, stream);
     if (p.epi == MOE_EPI_SWIGLU_BWD) return p.nn ? launch_variant<true, MOE_EPI_SWIGLU_BWD>(p, R, stream) : launch_variant<false, MOE_EPI_SWIGLU_BWD>(p, R, stream);
+    if (p.epi == MOE_EPI_SWIGLU_BWD_FUSED) {
+        if (p.nn || p.nrc != 3 || p.ncc != 2) return MOE_ERR_UNSUPPORTED;
+        for (int i = 0; i < 3; ++i) if (!p.RC[i] || !p.RCP[i] || (i < 2 && (!p.CB[i] || !p.CCP[i]))) return MOE_ERR_BAD_ARG;
+        return launch_variant<false, MOE_EPI_SWIGLU_BWD_FUSED>(p, R, stream);
+    }
     return MOE_ERR_BAD_ARG;
 }
 

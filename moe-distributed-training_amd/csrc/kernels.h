@@ -8,6 +8,7 @@
 #define MOE_EPI_STORE 0        // Y0[out_row][n] = acc
 #define MOE_EPI_SWIGLU 1       // weight pair (gate, up): Y0 = silu(gate)*up, optional Y1 = gate, Y2 = up (grouped rows)
 #define MOE_EPI_SWIGLU_BWD 2   // acc = dh: Y0 = dgate, Y1 = dup from saved gate (H1) and up (H3)
+#define MOE_EPI_SWIGLU_BWD_FUSED 3   // ... and the low-rank products of dgate, dup and h that the adapters' backward needs (RC / CB below)
 
 constexpr int MOE_MAX_SLABS = 4;
 
@@ -28,12 +29,18 @@ struct MoeGemmParams {
     const uint16_t* H1;     // saved gate / up for MOE_EPI_SWIGLU_BWD
     const uint16_t* H3;
     int64_t ldh;
-    // MOE_EPI_SWIGLU_BWD only: fused row contractions (nrc = 0 or 3).  RC[i]: bf16 [R][16] operands in grouped order;
+    // MOE_EPI_SWIGLU_BWD_FUSED only: row contractions (nrc = 3).  RC[i]: bf16 [R][16] operands in grouped order;
     // RCP[i]: fp32 partials [row tile][N][16], row tiles of 256 rows per expert in order (the layout the fixed-order
     // reduction of the adapter gradients sums): RCP[0] = dgate^T RC[0], RCP[1] = dup^T RC[1], RCP[2] = h^T RC[2]
     const uint16_t* RC[3];
     float* RCP[3];
     int nrc;
+    // ... and column contractions (ncc = 2): CB[i]: adapter factor in fragment order [E][N/32][64][8];
+    // CCP[i]: fp32 partials [column tile of 256][cc_rows][16]: CCP[0] = dgate CB[0], CCP[1] = dup CB[1] over the tile's columns
+    const uint16_t* CB[2];
+    float* CCP[2];
+    int ncc;
+    int64_t cc_rows;
     const float* row_scale; // optional per sorted position factor applied to the accumulator (STORE, SWIGLU_BWD)
     const void* pos;        // sorted_scattered_idxs
     int pos64;
@@ -110,6 +117,10 @@ int moe_launch_rows_lora2(const void* X, const void* X2, int64_t ldx, const void
                           int E, int64_t R, int64_t K, int fan_out, int x_grouped, float scaling,
                           const float* qt_row_scale, hipStream_t stream, void* q_scaled = nullptr);
 size_t moe_xtp_workspace_bytes(int64_t R, int E, int64_t K);
+// Q[m][r] = bf16(scaling * sum over ntiles column-tile partials [ntiles][R][16]) and its transposed copy Qt[r][m], for one or
+// two products (partial2 == nullptr: one)
+int moe_launch_cc_reduce2(const float* partial, const float* partial2, int ntiles, int64_t R, float scaling, void* Q, void* Q2,
+                          void* Qt, void* Qt2, int64_t ldqt, hipStream_t stream);
 // the reduction half of moe_launch_xtp2 alone, for partials [row tile of 256][K][16] that another kernel produced
 // (partial2 == nullptr: only the first)
 int moe_launch_xtp_reduce2(const float* partial, const float* partial2, void* out, void* out2, const int64_t* so,

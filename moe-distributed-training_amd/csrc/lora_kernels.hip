@@ -324,7 +324,34 @@ __global__ void xtp_reduce_kernel(const float* __restrict__ partial, int64_t par
     out[(int64_t)e * soe + k * sok + r * sor] = f32_to_bf16_bits(s * scale);
 }
 
+// Q[m][r] = bf16(scaling * sum_t partial[t][m][r]) (t ascending: a fixed order) and Qt[r][m] likewise
+__global__ void cc_reduce_kernel(const float* __restrict__ partial0, const float* __restrict__ partial1, int ntiles, int64_t R,
+                                 float scaling, uint16_t* __restrict__ Q0, uint16_t* __restrict__ Q1, uint16_t* __restrict__ Qt0,
+                                 uint16_t* __restrict__ Qt1, int64_t ldqt)
+{
+    const float* __restrict__ partial = blockIdx.y ? partial1 : partial0;
+    uint16_t* __restrict__ Q = blockIdx.y ? Q1 : Q0;
+    uint16_t* __restrict__ Qt = blockIdx.y ? Qt1 : Qt0;
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;   // (m, r) flattened
+    if (idx >= R * 16) return;
+    float s = 0.f;
+    for (int t = 0; t < ntiles; ++t) s += partial[(int64_t)t * R * 16 + idx];
+    const uint16_t v = f32_to_bf16_bits(s * scaling);
+    Q[idx] = v;
+    if (Qt) Qt[(idx & 15) * ldqt + (idx >> 4)] = v;
+}
+
 }  // namespace
+
+int moe_launch_cc_reduce2(const float* partial, const float* partial2, int ntiles, int64_t R, float scaling, void* Q, void* Q2,
+                          void* Qt, void* Qt2, int64_t ldqt, hipStream_t stream)
+{
+    if (R == 0) return MOE_OK;
+    const bool two = partial2 != nullptr;
+    hipLaunchKernelGGL(cc_reduce_kernel, dim3((unsigned)((R * 16 + 255) / 256), two ? 2u : 1u), dim3(256), 0, stream, partial, partial2,
+                       ntiles, R, scaling, (uint16_t*)Q, (uint16_t*)Q2, (uint16_t*)Qt, (uint16_t*)Qt2, ldqt);
+    return moe_launch_status();
+}
 
 int moe_launch_pack_lora(const void* src, int64_t se, int64_t sk, int64_t sr, void* dst, int E, int64_t K, int rank,
                          int transpose, hipStream_t stream)

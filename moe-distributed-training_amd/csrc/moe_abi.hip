@@ -408,6 +408,8 @@ static inline size_t sk_bytes_mlp(int64_t R, int E, int64_t d, int64_t f)
     const size_t a = moe_gemm_sk_bytes(R, E, d), b = moe_gemm_sk_bytes(R, E, f);
     return a > b ? a : b;
 }
+// column-tile partials of the two fused column contractions of the dh GEMM: [2][ceil(f / 256)][R][16] fp32
+static inline size_t cc_bytes(int64_t R, int64_t f) { return (size_t)2 * (size_t)((f + 255) / 256) * (size_t)R * 16 * sizeof(float); }
 static inline bool bad_pitch(int64_t ld) { return (ld * 2) % 4096 == 0; }
 static inline size_t repitch_bytes(int64_t R, int64_t d) { return al((size_t)R * (size_t)(d + 64) * 2); }
 
@@ -417,7 +419,7 @@ size_t moe_mlp_workspace_bytes(int64_t R, int E, int64_t d, int64_t f, int rank)
     if (rank <= 0) return n;
     const int64_t mx = d > f ? d : f;
     const size_t C = (size_t)(rank + 15) / 16;   // 16-wide chunks per adapter
-    return n + C * (3 * pack_bytes(E, d) + 3 * pack_bytes(E, f) + 7 * q_bytes(R)) + al(3 * moe_xtp_workspace_bytes(R, E, mx));
+    return n + C * (3 * pack_bytes(E, d) + 3 * pack_bytes(E, f) + 7 * q_bytes(R)) + al(3 * moe_xtp_workspace_bytes(R, E, mx)) + al(cc_bytes(R, f));
 }
 
 size_t moe_mlp_saved_bytes(int64_t R, int rank) { return rank > 0 ? (size_t)((rank + 15) / 16) * 6 * q_bytes(R) : 256; }
@@ -570,6 +572,7 @@ int moe_mlp_bwd(const void* dy, int64_t lddy, int dy_grouped, int dy_fan_out, co
     auto svp = [&](int which, int c) { return sv + ((size_t)c * 6 + which) * qb; };   // which: 0 Q1, 1 Q3, 2 Q2, 3 Qt1, 4 Qt3, 5 Qt2
     void* xw = nullptr;
     void* p2s = nullptr;
+    float* ccw = nullptr;
     size_t xb = 0;
     // a rank of at most 16 (one chunk): the adapter gradients that sum over the rows of dgate, dup and h are produced by
     // the dh GEMM's epilogue as per-row-tile partials; two chunks take the separate passes over those tensors
@@ -590,6 +593,7 @@ int moe_mlp_bwd(const void* dy, int64_t lddy, int dy_grouped, int dy_fan_out, co
     if (has_lora) {
         pq = (uint8_t*)ws.take((size_t)C * 6 * qb);
         if (fuse_rc) p2s = ws.take(qb);   // P2 times the row scale, row-major (the fused contraction's operand)
+        if (fuse_rc) ccw = (float*)ws.take(cc_bytes(R, f));
         const int64_t mx = d > f ? d : f;
         xb = 3 * moe_xtp_workspace_bytes(R, E, mx);   // paired reductions keep two sets of partials, the fused ones of the dh GEMM three
         xw = ws.take(xb);
@@ -644,6 +648,12 @@ int moe_mlp_bwd(const void* dy, int64_t lddy, int dy_grouped, int dy_fan_out, co
             p.RC[0] = (const uint16_t*)svp(0, 0); p.RC[1] = (const uint16_t*)svp(1, 0); p.RC[2] = (const uint16_t*)p2s;
             for (int i = 0; i < 3; ++i) p.RCP[i] = (float*)((uint8_t*)xw + i * one);
             p.nrc = 3;
+            // P1 = dgate B1^T, P3 = dup B3^T (the dX GEMM's low-rank operands) as per-column-tile partials
+            const size_t cone = cc_bytes(R, f) / 2 / sizeof(float);
+            p.CB[0] = (const uint16_t*)bt1[0]; p.CB[1] = (const uint16_t*)bt3[0];
+            p.CCP[0] = ccw; p.CCP[1] = ccw + cone;
+            p.ncc = 2; p.cc_rows = R;
+            p.epi = MOE_EPI_SWIGLU_BWD_FUSED;
         }
         moe_gemm_sk_attach(p, skws, R, E, f);
         p.counters_clean = counters_clean;
@@ -672,6 +682,10 @@ int moe_mlp_bwd(const void* dy, int64_t lddy, int dy_grouped, int dy_fan_out, co
                             rank < 16 ? rank : 16, C > 1 ? rank - 16 : 0, offsets, off64, E, R, d, 1.f, xw, xb, st)); }
         // ---- w1 / w3 backward
         TIMED("bwd.rows_lora_dgate_dup");
+        if (fuse_rc) {   // the products over each column tile came out of the dh GEMM's epilogue: add the tiles, scale, round
+            const size_t cone = cc_bytes(R, f) / 2 / sizeof(float);
+            TRY(moe_launch_cc_reduce2(ccw, ccw + cone, (int)((f + 255) / 256), R, scaling, pqp(1, 0), pqp(2, 0), pqp(4, 0), pqp(5, 0), ldt, st));
+        } else
         for (int c = 0; c < C; ++c)
             TRY(moe_launch_rows_lora2(dgate, dup, f, bt1[c], bt3[c], pqp(1, c), pqp(2, c), pqp(4, c), pqp(5, c), ldt, nullptr, 0, offsets,
                                       off64, E, R, f, 1, 1, scaling, nullptr, st));
