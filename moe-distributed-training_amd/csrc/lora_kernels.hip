@@ -296,7 +296,8 @@ __global__ void __launch_bounds__(XTP_THREADS) xtp_partial_kernel(const XtpJob j
         }
 }
 
-// out[e][k][r] = scale * sum over the expert's partial tiles (ascending), zero for an empty expert
+// out[e][k][r] = scale * sum over the expert's partial tiles (ascending), zero for an empty expert.  A thread owns four
+// consecutive rank columns of one k (one 16-byte load per tile, several tiles in flight).
 __global__ void xtp_reduce_kernel(const float* __restrict__ partial, int64_t partial_stride, const XtpJob job0,
                                   const XtpJob job1, const void* __restrict__ offsets, int off64,
                                   int E, int64_t K, float scale)
@@ -314,17 +315,31 @@ __global__ void xtp_reduce_kernel(const float* __restrict__ partial, int64_t par
         if (ee < e) tile0 += (end - start + XTP_RC - 1) / XTP_RC;
     }
     const int64_t ntile = (end - start + XTP_RC - 1) / XTP_RC;
-    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t idx = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
     if (idx >= K * 16) return;
     const int64_t k = idx >> 4;
     const int r = (int)(idx & 15);
-    if (r >= rank) return;
-    float s = 0.f;
-    for (int64_t t = 0; t < ntile; ++t) s += partial[(tile0 + t) * K * 16 + idx];
-    out[(int64_t)e * soe + k * sok + r * sor] = f32_to_bf16_bits(s * scale);
+    const float* __restrict__ src = partial + tile0 * K * 16 + idx;
+    f32x4_t s = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+    int64_t t = 0;
+    for (; t + 4 <= ntile; t += 4) {   // four loads in flight; the additions keep the ascending order
+        const f32x4_t a = *(const f32x4_t*)(src + (t + 0) * K * 16), b = *(const f32x4_t*)(src + (t + 1) * K * 16);
+        const f32x4_t c = *(const f32x4_t*)(src + (t + 2) * K * 16), d = *(const f32x4_t*)(src + (t + 3) * K * 16);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) s[q] = (((s[q] + a[q]) + b[q]) + c[q]) + d[q];
+    }
+    for (; t < ntile; ++t) {
+        const f32x4_t a = *(const f32x4_t*)(src + t * K * 16);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) s[q] += a[q];
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+        if (r + q < rank) out[(int64_t)e * soe + k * sok + (r + q) * sor] = f32_to_bf16_bits(s[q] * scale);
 }
 
-// Q[m][r] = bf16(scaling * sum_t partial[t][m][r]) (t ascending: a fixed order) and Qt[r][m] likewise
+// Q[m][r] = bf16(scaling * sum_t partial[t][m][r]) (t ascending: a fixed order) and Qt[r][m] likewise.  A thread owns
+// four consecutive rank columns of one row and keeps eight loads in flight.
 __global__ void cc_reduce_kernel(const float* __restrict__ partial0, const float* __restrict__ partial1, int ntiles, int64_t R,
                                  float scaling, uint16_t* __restrict__ Q0, uint16_t* __restrict__ Q1, uint16_t* __restrict__ Qt0,
                                  uint16_t* __restrict__ Qt1, int64_t ldqt)
@@ -332,13 +347,36 @@ __global__ void cc_reduce_kernel(const float* __restrict__ partial0, const float
     const float* __restrict__ partial = blockIdx.y ? partial1 : partial0;
     uint16_t* __restrict__ Q = blockIdx.y ? Q1 : Q0;
     uint16_t* __restrict__ Qt = blockIdx.y ? Qt1 : Qt0;
-    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;   // (m, r) flattened
+    const int64_t idx = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;   // (m, r) flattened, r a multiple of 4
     if (idx >= R * 16) return;
-    float s = 0.f;
-    for (int t = 0; t < ntiles; ++t) s += partial[(int64_t)t * R * 16 + idx];
-    const uint16_t v = f32_to_bf16_bits(s * scaling);
-    Q[idx] = v;
-    if (Qt) Qt[(idx & 15) * ldqt + (idx >> 4)] = v;
+    const float* __restrict__ src = partial + idx;
+    const int64_t step = R * 16;
+    f32x4_t s = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+    int t = 0;
+    for (; t + 8 <= ntiles; t += 8) {
+        f32x4_t v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = *(const f32x4_t*)(src + (int64_t)(t + u) * step);
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) s[q] += v[u][q];
+    }
+    for (; t < ntiles; ++t) {
+        const f32x4_t a = *(const f32x4_t*)(src + (int64_t)t * step);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) s[q] += a[q];
+    }
+    uint16_t o[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) o[q] = f32_to_bf16_bits(s[q] * scaling);
+    *(uint2*)(Q + idx) = make_uint2(o[0] | ((uint32_t)o[1] << 16), o[2] | ((uint32_t)o[3] << 16));
+    if (Qt) {
+        const int64_t m = idx >> 4;
+        const int r = (int)(idx & 15);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) Qt[(int64_t)(r + q) * ldqt + m] = o[q];
+    }
 }
 
 }  // namespace
@@ -348,7 +386,7 @@ int moe_launch_cc_reduce2(const float* partial, const float* partial2, int ntile
 {
     if (R == 0) return MOE_OK;
     const bool two = partial2 != nullptr;
-    hipLaunchKernelGGL(cc_reduce_kernel, dim3((unsigned)((R * 16 + 255) / 256), two ? 2u : 1u), dim3(256), 0, stream, partial, partial2,
+    hipLaunchKernelGGL(cc_reduce_kernel, dim3((unsigned)((R * 4 + 255) / 256), two ? 2u : 1u), dim3(256), 0, stream, partial, partial2,
                        ntiles, R, scaling, (uint16_t*)Q, (uint16_t*)Q2, (uint16_t*)Qt, (uint16_t*)Qt2, ldqt);
     return moe_launch_status();
 }
@@ -454,7 +492,7 @@ int moe_launch_xtp2(const void* X, const void* X2, int64_t ldx, const void* pos,
         hipLaunchKernelGGL(xtp_partial_kernel, grid, dim3(XTP_THREADS), 0, stream, j0, j1, ldx, pos, pos64, fan_out, ldpt,
                            p_row_scale, (float*)workspace, pstride, offsets, off64, E, R, K);
     }
-    dim3 rgrid((unsigned)((K * 16 + 255) / 256), (unsigned)E, two ? 2u : 1u);
+    dim3 rgrid((unsigned)((K * 4 + 255) / 256), (unsigned)E, two ? 2u : 1u);
     hipLaunchKernelGGL(xtp_reduce_kernel, rgrid, dim3(256), 0, stream, (const float*)workspace, pstride, j0, j1, offsets,
                        off64, E, K, scale);
     return moe_launch_status();
@@ -469,7 +507,7 @@ int moe_launch_xtp_reduce2(const float* partial, const float* partial2, void* ou
     if (rank < 1 || rank > 16 || (two && (rank2 < 1 || rank2 > 16))) return MOE_ERR_UNSUPPORTED;
     const XtpJob j0 = {nullptr, nullptr, (uint16_t*)out, so[0], so[1], so[2], rank};
     const XtpJob j1 = two ? XtpJob{nullptr, nullptr, (uint16_t*)out2, so2[0], so2[1], so2[2], rank2} : j0;
-    dim3 rgrid((unsigned)((K * 16 + 255) / 256), (unsigned)E, two ? 2u : 1u);
+    dim3 rgrid((unsigned)((K * 4 + 255) / 256), (unsigned)E, two ? 2u : 1u);
     hipLaunchKernelGGL(xtp_reduce_kernel, rgrid, dim3(256), 0, stream, partial, two ? (int64_t)(partial2 - partial) : 0, j0, j1,
                        offsets, off64, E, K, scale);
     return moe_launch_status();
