@@ -49,6 +49,10 @@ const char* moe_hip_strerror(int status);
  * moe_profile_get(i, ...) waits for record i and returns its stage name and device time in milliseconds.
  * This is the only process-wide state of the library and is off unless a harness turns it on. */
 int moe_profile_enable(int on);
+/* restricts the bracketing to stages whose name contains one of the comma-separated substrings (NULL or "": every
+ * stage).  A pair of events costs a few microseconds of device time, so a harness that times a whole step brackets only
+ * what it prices inside that region. */
+int moe_profile_select(const char* substrings);
 int moe_profile_count(void);
 int moe_profile_get(int i, char* name, int name_cap, float* ms);
 

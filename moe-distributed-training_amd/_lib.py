@@ -20,6 +20,7 @@ _SIGNATURES = {
     "moe_hip_abi_version": ("i", ""),
     "moe_hip_strerror": ("s", "i"),
     "moe_profile_enable": ("i", "i"),
+    "moe_profile_select": ("i", "p"),
     "moe_profile_count": ("i", ""),
     "moe_profile_get": ("i", "ipip"),
     "moe_router_logits": ("i", "plplipllip"),

@@ -4,6 +4,7 @@
 #include "common.h"
 #include "kernels.h"
 #include <mutex>
+#include <string>
 #include <string.h>
 #include <stdlib.h>
 #include <vector>
@@ -16,6 +17,7 @@ namespace {
 struct ProfRec { const char* name; hipEvent_t a, b; };
 std::mutex g_prof_mu;
 bool g_prof_on = false;
+std::string g_prof_select;   // comma-separated substrings; empty = every stage
 std::vector<ProfRec> g_prof;
 std::vector<hipEvent_t> g_prof_pool;
 
@@ -24,6 +26,17 @@ struct Timed {
     Timed(hipStream_t s, const char* name) : st(s), b(nullptr), on(false) {
         std::lock_guard<std::mutex> lk(g_prof_mu);
         if (!g_prof_on) return;
+        if (!g_prof_select.empty()) {   // only the selected stages are bracketed
+            bool hit = false;
+            size_t a = 0;
+            while (a <= g_prof_select.size() && !hit) {
+                size_t b = g_prof_select.find(',', a);
+                if (b == std::string::npos) b = g_prof_select.size();
+                if (b > a && strstr(name, g_prof_select.substr(a, b - a).c_str())) hit = true;
+                a = b + 1;
+            }
+            if (!hit) return;
+        }
         hipEvent_t ev[2];
         for (int i = 0; i < 2; ++i) {
             if (!g_prof_pool.empty()) { ev[i] = g_prof_pool.back(); g_prof_pool.pop_back(); }
@@ -67,6 +80,13 @@ int moe_profile_enable(int on)
     for (auto& r : g_prof) { g_prof_pool.push_back(r.a); g_prof_pool.push_back(r.b); }
     g_prof.clear();
     g_prof_on = on != 0;
+    return MOE_OK;
+}
+
+int moe_profile_select(const char* substrings)
+{
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    g_prof_select = substrings ? substrings : "";
     return MOE_OK;
 }
 
