@@ -355,6 +355,9 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
     // number of 16-row MFMA blocks of this wave that hold at least one real row
     int mb_cnt = (nrows - wm * WTM + 15) / 16;
     mb_cnt = mb_cnt < 0 ? 0 : (mb_cnt > MB ? MB : mb_cnt);
+    // the same in every lane: as a scalar, the checks around the MFMAs of a ragged tile are scalar branches (under a
+    // vector condition the compiler masks single MFMAs instead of branching around them, and the matrix cores ignore the mask)
+    mb_cnt = __builtin_amdgcn_readfirstlane(mb_cnt);
 
     const int kb = ktiles * part / nparts;
     const int ke = ktiles * (part + 1) / nparts;

@@ -6,7 +6,6 @@
 #include <mutex>
 #include <string>
 #include <string.h>
-#include <stdlib.h>
 #include <vector>
 
 namespace {
@@ -596,7 +595,7 @@ int moe_mlp_bwd(const void* dy, int64_t lddy, int dy_grouped, int dy_fan_out, co
     size_t xb = 0;
     // a rank of at most 16 (one chunk): the adapter gradients that sum over the rows of dgate, dup and h are produced by
     // the dh GEMM's epilogue as per-row-tile partials; two chunks take the separate passes over those tensors
-    const bool fuse_rc = has_lora && rank <= 16 && getenv("MOE_NO_FUSE_RC") == nullptr;
+    const bool fuse_rc = has_lora && rank <= 16;
     if (!workspace || workspace_bytes < moe_mlp_workspace_bytes(R, E, d, f, has_lora ? rank : 0)) return MOE_ERR_WORKSPACE;
     Bump ws(workspace, workspace_bytes);
     void* skws = ws.take(sk_bytes_mlp(R, E, d, f));
