@@ -22,6 +22,7 @@
 #ifndef SK_ORDER
 #define SK_ORDER __ATOMIC_ACQ_REL
 #endif
+#define EPI_IS_PAIR(e) ((e) == MOE_EPI_SWIGLU || (e) == MOE_EPI_SWIGLU_FUSED)
 constexpr int NXCD_HOST = 8;
 static int moe_num_cus()
 {
@@ -225,7 +226,7 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
 
     // ---- work item -> (expert, n tile, m tile, K part)
-    const int ntiles_n = (EPI == MOE_EPI_SWIGLU) ? (int)((p.N + BN / 2 - 1) / (BN / 2)) : (int)((p.N + BN - 1) / BN);
+    const int ntiles_n = (EPI_IS_PAIR(EPI)) ? (int)((p.N + BN / 2 - 1) / (BN / 2)) : (int)((p.N + BN - 1) / BN);
     const int ktiles_seg = (int)(p.K / BK);
     const int ktiles = ktiles_seg * p.nseg;
     const WorkItem item = decode_work_item(p.offsets, p.off64, p.E, ntiles_n, ktiles, p.max_split, p.num_cus);
@@ -233,7 +234,7 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
     const int expert = item.expert, nt = item.nt, part = item.part, nparts = item.nparts, split_item = item.split_item;
     const int64_t row0 = item.row0, row1 = item.row1;
     const int nrows = (int)(row1 - row0);
-    const int64_t n0 = (int64_t)nt * ((EPI == MOE_EPI_SWIGLU) ? BN / 2 : BN);
+    const int64_t n0 = (int64_t)nt * ((EPI_IS_PAIR(EPI)) ? BN / 2 : BN);
 
     // ---- row tables
     for (int r = tid; r < BM; r += NTHREADS) {
@@ -275,7 +276,7 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
         for (int j = 0; j < LPT; ++j) {
             const int r = (j * NWAVES + wave) * 8 + (lane >> 3);
             const int c = (lane & 7) ^ ((r >> 1) & 7);
-            int64_t n = (EPI == MOE_EPI_SWIGLU) ? n0 + (r & (BN / 2 - 1)) : n0 + r;
+            int64_t n = (EPI_IS_PAIR(EPI)) ? n0 + (r & (BN / 2 - 1)) : n0 + r;
             if (n >= p.N) n = p.N - 1;
             b_off[j] = (uint32_t)((n * p.ldw + c * 8) * 2);
         }
@@ -313,7 +314,7 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
             const int i = wave * 32 + (lane >> 1);
             const int r = i < nrows ? i : nrows - 1;
             slab_off_q = (uint32_t)((r * 16 + (lane & 1) * 8) * 2);             // + row0 * 32 as the scalar offset
-            int64_t n = (EPI == MOE_EPI_SWIGLU) ? n0 + (i & (BN / 2 - 1)) : n0 + i;
+            int64_t n = (EPI_IS_PAIR(EPI)) ? n0 + (i & (BN / 2 - 1)) : n0 + i;
             if (n >= p.N) n = p.N - 1;
             slab_off_l = (uint32_t)(((n - n0) * 16 + (lane & 1) * 8) * 2);      // + n0 * 32
         }
@@ -387,7 +388,7 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
         kt = __builtin_amdgcn_readfirstlane(kt < ke ? kt : ke - 1);
         const int seg = (kt >= ktiles_seg) ? 1 : 0;
         const uint32_t k0 = (uint32_t)(kt - seg * ktiles_seg) * BK;
-        const bool second = (EPI == MOE_EPI_SWIGLU) ? (idx >= LPT / 2) : (seg != 0);
+        const bool second = (EPI_IS_PAIR(EPI)) ? (idx >= LPT / 2) : (seg != 0);
         load_to_lds_16(second ? b_buf1 : b_buf0, b_off[idx], NN ? k0 * (uint32_t)p.ldw * 2 : k0 * 2, smem_u + B_REGION + stage * B_STAGE_BYTES + idx * (NWAVES * 1024));
     };
 
@@ -395,7 +396,7 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
     // MFMA's first operand -- so that a lane ends up with 4 consecutive output columns of one row (8-byte packs).
     auto read_b1 = [&](const uint8_t* b_lds, int ks, int nb, bf16x8_t* bfrag) {
         if (!NN) {
-            const int brow = (EPI == MOE_EPI_SWIGLU) ? (nb / NBH) * (BN / 2) + wn * (WTN / 2) + (nb % NBH) * 16 : wn * WTN + nb * 16;
+            const int brow = (EPI_IS_PAIR(EPI)) ? (nb / NBH) * (BN / 2) + wn * (WTN / 2) + (nb % NBH) * 16 : wn * WTN + nb * 16;
             bfrag[nb] = *(const bf16x8_t*)(b_lds + brow * 128 + b_frag_off[ks]);
         } else {
             const uint8_t* bp = b_lds + b_frag_off[nb] + ks * 32 * (BN / 8) * 16;
@@ -493,7 +494,8 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
                         const int nbr = ((nhs & 1) == 0) ? NB : 0;   // weight fragments first, when a new k step starts
                         const int q = m / READ_GAP;
                         if (q < nbr) { read_b1(rb, nhs >> 1, q, bf[cur_b ^ 1]); __builtin_amdgcn_sched_barrier(0); }
-                        else if (q - nbr < MBH) { read_a1(ra, nhs >> 1, nhs & 1, q - nbr, af[cur_a ^ 1]); __builtin_amdgcn_sched_barrier(0); }
+                        // (a ragged tile does not fetch the fragments of row blocks without real rows: its MFMAs on them are skipped too)
+                        else if (q - nbr < MBH) { if (FULL || (nhs & 1) * MBH + (q - nbr) < mb_cnt) read_a1(ra, nhs >> 1, nhs & 1, q - nbr, af[cur_a ^ 1]); __builtin_amdgcn_sched_barrier(0); }
                     }
                     if (hs == 3 && m % A_LOAD_GAP == 0 && m / A_LOAD_GAP < LPT) {
                         if (SLAB) issue_slab(m / A_LOAD_GAP, as); else issue_a(kt + 2, m / A_LOAD_GAP, as, !FULL);
@@ -607,7 +609,7 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
                     const uint8_t* img = smem + ((ke - kb) & 1) * A_STAGE_BYTES + src * (BM * 32) + 16 * kc;
 #pragma unroll
                     for (int nb = 0; nb < NB; ++nb) {
-                        const int c = (EPI == MOE_EPI_SWIGLU) ? wn * (WTN / 2) + (nb % NBH) * 16 + (lane & 15) : wn * WTN + nb * 16 + (lane & 15);
+                        const int c = (EPI_IS_PAIR(EPI)) ? wn * (WTN / 2) + (nb % NBH) * 16 + (lane & 15) : wn * WTN + nb * 16 + (lane & 15);
                         bf16x8_t v = {};
                         if (live) v = *(const bf16x8_t*)(img + 2 * (BM * 32) + c * 32);
                         sb[s][nb] = v;
@@ -624,7 +626,7 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
                 const uint16_t* LB = p.LB[src] + (int64_t)expert * p.N * 16;
 #pragma unroll
                 for (int nb = 0; nb < NB; ++nb) {
-                    int64_t n = (EPI == MOE_EPI_SWIGLU) ? n0 + wn * (WTN / 2) + (nb % NBH) * 16 + (lane & 15) : n0 + wn * WTN + nb * 16 + (lane & 15);
+                    int64_t n = (EPI_IS_PAIR(EPI)) ? n0 + wn * (WTN / 2) + (nb % NBH) * 16 + (lane & 15) : n0 + wn * WTN + nb * 16 + (lane & 15);
                     if (n >= p.N) n = p.N - 1;
                     bf16x8_t v = {};
                     if (live) v = *(const bf16x8_t*)(LB + n * 16 + 8 * kc);
@@ -727,7 +729,7 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
                 stage_put(WTN, mb * 16 + mrow, nb * 16 + nq, pack4(acc[mb][nb][0] * s_, acc[mb][nb][1] * s_, acc[mb][nb][2] * s_, acc[mb][nb][3] * s_));
             }
         stage_flush(WTN, p.Y[0], p.ldy, !p.y_grouped, n0 + wn * WTN);
-    } else if (EPI == MOE_EPI_SWIGLU) {
+    } else if (EPI_IS_PAIR(EPI)) {
         // gate = acc[mb][j], up = acc[mb][NBH + j] at identical (row, column) positions; both are rounded to storage
         // precision first (in place) so that forward and backward see the same values
         const int64_t ncol0 = n0 + wn * (WTN / 2);
@@ -758,7 +760,48 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
                     }
                     stage_put(WTN / 2, mb * 16 + mrow, nj * 16 + nq, pack4(o[0], o[1], o[2], o[3]));
                 }
+            if (EPI == MOE_EPI_SWIGLU_FUSED && pass == 0) {
+                // Fused column contraction (the low-rank interim of the next GEMM): CCP[0][nt][m][r] = sum_n h[m][n] CB[0][e][n][r]
+                // over this tile's 128 columns of h, from the staged image of h (read row-major: the contraction index is the
+                // column; this wave's 32 columns are one MFMA step), so that h is not read from memory again for it.  CB is the
+                // adapter factor in MFMA fragment order.  The wave parks its sums in the free half of its staging slot.
+                const int64_t hcol = n0 + wn * (WTN / 2);
+                bf16x8_t cb = {};
+                if (hcol < p.N) cb = *(const bf16x8_t*)(p.CB[0] + ((int64_t)expert * p.N + hcol) * 16 + lane * 8);
+                float* park = (float*)(stg + WTM * (WTN / 2) * 2);
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb) {
+                    const bf16x8_t hf = *(const bf16x8_t*)(stg + (mb * 16 + (lane & 15)) * (WTN / 2 * 2) + (((lane >> 4) ^ ((lane >> 2) & 3)) << 4));
+                    const f32x4_t z = {0.f, 0.f, 0.f, 0.f};
+                    const f32x4_t d_ = __builtin_amdgcn_mfma_f32_16x16x32_bf16(hf, cb, z, 0, 0, 0);
+                    *(f32x4_t*)(park + (mb * 64 + lane) * 4) = d_;
+                }
+            }
             stage_flush(WTN / 2, Y, p.ldy, false, ncol0);
+        }
+        if (EPI == MOE_EPI_SWIGLU_FUSED) {
+            // element (row = mb*16 + 4*(lane/16) + reg, rank column lane%16) of every column wave's sums is parked in its slot;
+            // wave (wm, wn) adds the four column waves' sums (in wave order) of row blocks 2 wn, 2 wn + 1 and stores them
+            __builtin_amdgcn_s_waitcnt(0xC07F);
+            __syncthreads();
+            const int tg = lane >> 4, ti = lane & 15;
+#pragma unroll
+            for (int h2 = 0; h2 < 2; ++h2) {
+                const int mb = 2 * wn + h2;
+                f32x4_t sum = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int w2 = 0; w2 < WAVES_N; ++w2) {
+                    const float* src = (const float*)(smem + (wm * WAVES_N + w2) * (WTM * WTN * 2) + WTM * (WTN / 2) * 2);
+                    const f32x4_t v = *(const f32x4_t*)(src + (mb * 64 + lane) * 4);
+#pragma unroll
+                    for (int reg = 0; reg < 4; ++reg) sum[reg] += v[reg];
+                }
+                const int rl0 = wm * WTM + mb * 16 + 4 * tg;
+                float* dst = p.CCP[0] + ((int64_t)nt * p.cc_rows + row0 + rl0) * 16 + ti;
+#pragma unroll
+                for (int reg = 0; reg < 4; ++reg)
+                    if (rl0 + reg < nrows) dst[reg * 16] = sum[reg];
+            }
         }
     } else {  // MOE_EPI_SWIGLU_BWD: acc = dh; dgate = dh * up * sig(g) * (1 + g (1 - sig(g))), dup = dh * silu(g)
         // dh (scaled by the row's routing weight) is staged as bf16 -- the precision a stored dh would have -- and
@@ -1045,11 +1088,11 @@ template <bool NN, int EPI> int launch_variant(const MoeGemmParams& p, int64_t R
             return MOE_ERR_LAUNCH;
         attr_set = true;
     }
-    const int ntiles_n = (EPI == MOE_EPI_SWIGLU) ? (int)((p.N + BN / 2 - 1) / (BN / 2)) : (int)((p.N + BN - 1) / BN);
+    const int ntiles_n = (EPI_IS_PAIR(EPI)) ? (int)((p.N + BN / 2 - 1) / (BN / 2)) : (int)((p.N + BN - 1) / BN);
     MoeGemmParams q = p;
     q.num_cus = moe_num_cus();
     q.y_wide = (!p.y_grouped && (R * p.ldy + p.N) * 2 >= ((int64_t)1 << 31)) ? 1 : 0;
-    q.max_split = moe_gemm_max_split(EPI == MOE_EPI_SWIGLU);
+    q.max_split = moe_gemm_max_split(EPI_IS_PAIR(EPI));
     if (q.max_split > 1) {
         if (!p.sk_partials || !p.sk_counters) return MOE_ERR_WORKSPACE;
         if (!p.counters_clean) hipLaunchKernelGGL(zero_i32_kernel, dim3((unsigned)((q.num_cus + 255) / 256)), dim3(256), 0, stream, p.sk_counters, (int64_t)q.num_cus);
@@ -1123,6 +1166,11 @@ int moe_launch_gemm_mfma(const MoeGemmParams& p, int64_t R, hipStream_t stream)
     if (!moe_gemm_mfma_supported(p, R)) return MOE_ERR_UNSUPPORTED;
     if (p.epi == MOE_EPI_STORE) return p.nn ? launch_variant<true, MOE_EPI_STORE>(p, R, stream) : launch_variant<false, MOE_EPI_STORE>(p, R, stream);
     if (p.epi == MOE_EPI_SWIGLU) return p.nn ? MOE_ERR_UNSUPPORTED : launch_variant<false, MOE_EPI_SWIGLU>(p, R, stream);
+    if (p.epi == MOE_EPI_SWIGLU_FUSED) {
+        if (p.nn || p.ncc != 1) return MOE_ERR_UNSUPPORTED;
+        if (!p.CB[0] || !p.CCP[0] || !p.Y[0]) return MOE_ERR_BAD_ARG;
+        return launch_variant<false, MOE_EPI_SWIGLU_FUSED>(p, R, stream);
+    }
     if (p.epi == MOE_EPI_SWIGLU_BWD) return p.nn ? launch_variant<true, MOE_EPI_SWIGLU_BWD>(p, R, stream) : launch_variant<false, MOE_EPI_SWIGLU_BWD>(p, R, stream);
     if (p.epi == MOE_EPI_SWIGLU_BWD_FUSED) {
         if (p.nn || p.nrc != 3 || p.ncc != 2) return MOE_ERR_UNSUPPORTED;

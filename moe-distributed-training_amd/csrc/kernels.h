@@ -8,6 +8,7 @@
 #define MOE_EPI_STORE 0        // Y0[out_row][n] = acc
 #define MOE_EPI_SWIGLU 1       // weight pair (gate, up): Y0 = silu(gate)*up, optional Y1 = gate, Y2 = up (grouped rows)
 #define MOE_EPI_SWIGLU_BWD 2   // acc = dh: Y0 = dgate, Y1 = dup from saved gate (H1) and up (H3)
+#define MOE_EPI_SWIGLU_FUSED 4   // as MOE_EPI_SWIGLU, and the product of h with an adapter factor per column tile (CB[0] -> CCP[0], ncc = 1)
 #define MOE_EPI_SWIGLU_BWD_FUSED 3   // ... and the low-rank products of dgate, dup and h that the adapters' backward needs (RC / CB below)
 
 constexpr int MOE_MAX_SLABS = 4;
@@ -35,7 +36,7 @@ struct MoeGemmParams {
     const uint16_t* RC[3];
     float* RCP[3];
     int nrc;
-    // ... and column contractions (ncc = 2): CB[i]: adapter factor in fragment order [E][N/32][64][8];
+    // ... and column contractions (MOE_EPI_SWIGLU_BWD_FUSED: ncc = 2; MOE_EPI_SWIGLU_FUSED: ncc = 1, CCP[0] = h CB[0] per column tile of 128): CB[i]: adapter factor in fragment order [E][N/32][64][8];
     // CCP[i]: fp32 partials [column tile of 256][cc_rows][16]: CCP[0] = dgate CB[0], CCP[1] = dup CB[1] over the tile's columns
     const uint16_t* CB[2];
     float* CCP[2];

@@ -490,6 +490,11 @@ int moe_mlp_fwd(const void* x, int64_t ldx, const void* w1, const void* w3, cons
     const int C = has_lora ? (rank + 15) / 16 : 0;
     auto svp = [&](int which, int c) { return sv + ((size_t)c * 6 + which) * qb; };   // which: 0 Q1, 1 Q3, 2 Q2, 3 Qt1, 4 Qt3, 5 Qt2
     void *At1[2] = {}, *At3[2] = {}, *lb1[2] = {}, *lb3[2] = {}, *At2c[2] = {}, *lb2[2] = {};
+    // a rank of at most 16: the w2 GEMM's low-rank operand Q2 = h A2 comes out of the pair GEMM's epilogue as per-column-tile
+    // partials (h is not read again for it); two chunks take the separate pass over h
+    const bool fuse_q2 = has_lora && rank <= 16;
+    float* ccw = fuse_q2 ? (float*)ws.take(cc_bytes(R, f)) : nullptr;
+    if (fuse_q2 && !ccw) return MOE_ERR_WORKSPACE;
     if (has_lora) {
         // lora order a1,b1,a3,b3,a2,b2; strides {expert, dim1, dim2}
         { TIMED("fwd.pack_lora");
@@ -532,14 +537,21 @@ int moe_mlp_fwd(const void* x, int64_t ldx, const void* w1, const void* w3, cons
         p.Y[0] = (uint16_t*)h; p.Y[1] = (uint16_t*)gate; p.Y[2] = (uint16_t*)up; p.ldy = f;
         p.pos = pos; p.pos64 = pos64; p.offsets = offsets; p.off64 = off64;
         p.E = E; p.K = d; p.N = f; p.fan_out = fan_out; p.x_grouped = 0; p.y_grouped = 1; p.epi = MOE_EPI_SWIGLU;
+        if (fuse_q2) {   // Q2 = h A2 (the w2 GEMM's low-rank operand) as per-column-tile partials from the epilogue
+            p.epi = MOE_EPI_SWIGLU_FUSED;
+            p.CB[0] = (const uint16_t*)At2c[0]; p.CCP[0] = ccw; p.ncc = 1; p.cc_rows = R;
+        }
         moe_gemm_sk_attach(p, skws, R, E, f);
         p.counters_clean = counters_clean;
-        if (moe_gemm_max_split(p.epi == MOE_EPI_SWIGLU) > 1) counters_clean = true;   // zeroed by that launch if they were not, and left zero
+        if (moe_gemm_max_split(p.epi == MOE_EPI_SWIGLU || p.epi == MOE_EPI_SWIGLU_FUSED) > 1) counters_clean = true;   // zeroed by that launch if they were not, and left zero
         TIMED("fwd.gemm_w1w3_swiglu");
         TRY(moe_launch_gemm_mfma(p, R, st));
     }
     if (has_lora) {
         TIMED("fwd.rows_lora_h");
+        if (fuse_q2)   // the products over each column tile came out of the pair GEMM's epilogue: add the tiles, scale, round
+            TRY(moe_launch_cc_reduce2(ccw, nullptr, (int)((f + 127) / 128), R, scaling, svp(2, 0), nullptr, svp(5, 0), nullptr, ldt, st));
+        else
         TRY(moe_launch_rows_lora2(h, C > 1 ? h : nullptr, f, At2c[0], At2c[1], svp(2, 0), C > 1 ? svp(2, 1) : nullptr, svp(5, 0),
                                   C > 1 ? svp(5, 1) : nullptr, ldt, nullptr, 0, offsets, off64, E, R, f, 1, 1, scaling, nullptr, st));
     }
@@ -556,7 +568,7 @@ int moe_mlp_fwd(const void* x, int64_t ldx, const void* w1, const void* w3, cons
         p.E = E; p.K = f; p.N = d; p.fan_out = 1; p.x_grouped = 1; p.y_grouped = y_grouped; p.epi = MOE_EPI_STORE;
         moe_gemm_sk_attach(p, skws, R, E, d);
         p.counters_clean = counters_clean;
-        if (moe_gemm_max_split(p.epi == MOE_EPI_SWIGLU) > 1) counters_clean = true;   // zeroed by that launch if they were not, and left zero
+        if (moe_gemm_max_split(p.epi == MOE_EPI_SWIGLU || p.epi == MOE_EPI_SWIGLU_FUSED) > 1) counters_clean = true;   // zeroed by that launch if they were not, and left zero
         TIMED("fwd.gemm_w2");
         TRY(moe_launch_gemm_mfma(p, R, st));
     }
@@ -676,7 +688,7 @@ int moe_mlp_bwd(const void* dy, int64_t lddy, int dy_grouped, int dy_fan_out, co
         }
         moe_gemm_sk_attach(p, skws, R, E, f);
         p.counters_clean = counters_clean;
-        if (moe_gemm_max_split(p.epi == MOE_EPI_SWIGLU) > 1) counters_clean = true;   // zeroed by that launch if they were not, and left zero
+        if (moe_gemm_max_split(p.epi == MOE_EPI_SWIGLU || p.epi == MOE_EPI_SWIGLU_FUSED) > 1) counters_clean = true;   // zeroed by that launch if they were not, and left zero
         TIMED("bwd.gemm_dh_swiglu_bwd");
         TRY(moe_launch_gemm_mfma(p, R, st));
     }
@@ -725,7 +737,7 @@ int moe_mlp_bwd(const void* dy, int64_t lddy, int dy_grouped, int dy_fan_out, co
         p.E = E; p.K = f; p.N = d; p.fan_out = 1; p.x_grouped = 1; p.y_grouped = dx_grouped; p.epi = MOE_EPI_STORE;
         moe_gemm_sk_attach(p, skws, R, E, d);
         p.counters_clean = counters_clean;
-        if (moe_gemm_max_split(p.epi == MOE_EPI_SWIGLU) > 1) counters_clean = true;   // zeroed by that launch if they were not, and left zero
+        if (moe_gemm_max_split(p.epi == MOE_EPI_SWIGLU || p.epi == MOE_EPI_SWIGLU_FUSED) > 1) counters_clean = true;   // zeroed by that launch if they were not, and left zero
         TIMED("bwd.gemm_dx_w1w3");
         TRY(moe_launch_gemm_mfma(p, R, st));
     }
