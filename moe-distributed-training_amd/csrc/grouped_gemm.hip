@@ -429,7 +429,14 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
     // stage just freed), the two after that weight tile kt+3 (into the B stage just freed).  The next barrier then only
     // has to see the activation loads -- requested first, mostly cache hits -- and the weight tile requested a whole
     // tile earlier: the youngest LPT loads, weight loads that may well be waiting for HBM, stay in flight across it.
-    auto mainloop = [&](auto full_tag) {
+    // NBLK: how many of the wave's MB 16-row blocks take part -- MB for every wave of a full tile; in a ragged tile each
+    // wave runs the copy of the loop that fits its own rows, the count of its live blocks rounded up to 0, 1, 2, MBH or MB
+    // (0: no MFMAs, no fragment reads, the wave only issues its loads and meets the barriers).  A compile-time count, not a
+    // check per block: a check is a scalar branch per MFMA, and a tail tile of a few rows spent more time on those branches
+    // than on its MFMAs.  Blocks inside the count that lie past the group work on whatever their LDS rows hold (rows past
+    // the last 32-row block are never loaded); every consumer of the accumulators masks rows past the group.
+    auto mainloop = [&](auto nblk_tag, auto full_tag) {
+        constexpr int NBLK = decltype(nblk_tag)::value;
         constexpr bool FULL = decltype(full_tag)::value;
 #pragma unroll
         for (int i = 0; i < LPT; ++i) issue_a(kb, i, 0, !FULL);
@@ -496,9 +503,9 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
                     if (m % READ_GAP == 0) {
                         const int nbr = ((nhs & 1) == 0) ? NB : 0;   // weight fragments first, when a new k step starts
                         const int q = m / READ_GAP;
-                        if (q < nbr) { read_b1(rb, nhs >> 1, q, bf[cur_b ^ 1]); __builtin_amdgcn_sched_barrier(0); }
-                        // (a ragged tile does not fetch the fragments of row blocks without real rows: its MFMAs on them are skipped too)
-                        else if (q - nbr < MBH) { if (FULL || (nhs & 1) * MBH + (q - nbr) < mb_cnt) read_a1(ra, nhs >> 1, nhs & 1, q - nbr, af[cur_a ^ 1]); __builtin_amdgcn_sched_barrier(0); }
+                        if (q < nbr) { if (NBLK > 0) read_b1(rb, nhs >> 1, q, bf[cur_b ^ 1]); __builtin_amdgcn_sched_barrier(0); }
+                        // (a wave does not fetch the fragments of row blocks beyond its count: its MFMAs on them are skipped too)
+                        else if (q - nbr < MBH) { if ((nhs & 1) * MBH + (q - nbr) < NBLK) read_a1(ra, nhs >> 1, nhs & 1, q - nbr, af[cur_a ^ 1]); __builtin_amdgcn_sched_barrier(0); }
                     }
                     if (hs == 3 && m % A_LOAD_GAP == 0 && m / A_LOAD_GAP < LPT) {
                         if (SLAB) issue_slab(m / A_LOAD_GAP, as); else issue_a(kt + 2, m / A_LOAD_GAP, as, !FULL);
@@ -509,7 +516,7 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
                         issue_b(kt + 2, gb / B_LOAD_GAP, bs2);
                         __builtin_amdgcn_sched_barrier(0);
                     }
-                    if (FULL || mh * MBH + mb < mb_cnt)
+                    if (mh * MBH + mb < NBLK)
                         acc[mh * MBH + mb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bf[cur_b][nb], af[cur_a][mb], acc[mh * MBH + mb][nb], 0, 0, 0);
                 }
                 __builtin_amdgcn_s_setprio(0);
@@ -527,8 +534,14 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
         __builtin_amdgcn_s_waitcnt(0x0F70);   // loads past the last tile must not land in the epilogue's staging
         __syncthreads();   // operand buffers are free for the epilogue staging
     };
-    // full tiles run a loop body without any checks; a wave of a ragged tile checks its MFMA blocks and A loads
-    if (live_rows == BM) mainloop(std::true_type{}); else mainloop(std::false_type{});
+    // full tiles run a loop body without any checks; in a ragged tile the activation loads of dead row blocks are dropped
+    // and every wave takes the loop for the number of its live blocks (a scalar: the same in all lanes of the wave)
+    if (live_rows == BM) mainloop(std::integral_constant<int, MB>{}, std::true_type{});
+    else if (mb_cnt > MBH) mainloop(std::integral_constant<int, MB>{}, std::false_type{});
+    else if (mb_cnt > 2) mainloop(std::integral_constant<int, MBH>{}, std::false_type{});
+    else if (mb_cnt == 2) mainloop(std::integral_constant<int, 2>{}, std::false_type{});
+    else if (mb_cnt == 1) mainloop(std::integral_constant<int, 1>{}, std::false_type{});
+    else mainloop(std::integral_constant<int, 0>{}, std::false_type{});
     if (!p.y_grouped) {   // the output row table again: weight tiles have passed through its place
         for (int r = tid; r < BM; r += NTHREADS) s_outrow[r] = load_idx(p.pos, row0 + ((r < nrows) ? r : nrows - 1), p.pos64);
         __syncthreads();
