@@ -459,6 +459,16 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
 #pragma unroll
         for (int mb = 0; mb < MBH; ++mb) read_a1(smem, 0, 0, mb, af[0]);
         int bs = 0;   // B stage of tile kt
+        // A tail tile of at most two row blocks has next to no MFMA work and would run through K several times faster than
+        // the full row tiles that share its weight tiles: the weight tiles it fetches are then gone from L2 again before
+        // those arrive, and its requests compete with theirs.  Its waves therefore take at least PACE_CYCLES per K tile (a
+        // full tile cannot take less: 2048 cycles are its MFMAs alone), which keeps it just ahead of them -- close enough
+        // to act as their prefetcher.  Measured over nine routing draws of 8192 rows: the GEMM launches other than the
+        // gate/up pair 1-2 % faster; the pair launch, with sixteen rounds of tiles, is bound by the sum of its tiles' times
+        // and runs slower with paced tails, so it is left alone.
+        constexpr bool PACED = !FULL && NBLK <= 2 && !(EPI_IS_PAIR(EPI));
+        constexpr int64_t PACE_CYCLES = 2048;
+        int64_t pace_t0 = PACED ? (int64_t)__builtin_readcyclecounter() : 0;
         // one K tile; SLAB: the activation loads it requests (for tile kt+2) fetch the slab image instead
         auto tile = [&](int kt, auto slab_tag) {
             constexpr bool SLAB = decltype(slab_tag)::value;
@@ -474,6 +484,10 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
                 // ra / rb: where the fragments of the next half step come from; for the last one of a tile, the first of
                 // the next tile.  (After the last tile this fetches fragments nobody uses.)
                 if (hs == 3) {
+                    if (PACED) {   // (see PACE_CYCLES)
+                        while ((int64_t)__builtin_readcyclecounter() - pace_t0 < PACE_CYCLES) __builtin_amdgcn_s_sleep(2);
+                        pace_t0 = (int64_t)__builtin_readcyclecounter();
+                    }
                     __builtin_amdgcn_s_waitcnt(0x0F70 | LPT);   // all but the youngest LPT loads: tile kt+1 has landed
                     __syncthreads();                            // for every wave; and every wave is done reading tile kt
                 }
