@@ -463,7 +463,7 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
         // the full row tiles that share its weight tiles: the weight tiles it fetches are then gone from L2 again before
         // those arrive, and its requests compete with theirs.  Its waves therefore take at least PACE_CYCLES per K tile (a
         // full tile cannot take less: 2048 cycles are its MFMAs alone), which keeps it just ahead of them -- close enough
-        // to act as their prefetcher.  Measured over nine routing draws of 8192 rows: the GEMM launches other than the
+        // to act as their prefetcher.  Measured over eight routing draws of 8192 rows: the GEMM launches other than the
         // gate/up pair 1-2 % faster; the pair launch, with sixteen rounds of tiles, is bound by the sum of its tiles' times
         // and runs slower with paced tails, so it is left alone.
         constexpr bool PACED = !FULL && NBLK <= 2 && !(EPI_IS_PAIR(EPI));
