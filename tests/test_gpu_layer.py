@@ -443,6 +443,45 @@ def test_skewed_routing_and_ep_share(dev, oracle):
     assert torch.equal(ei_sub, ei[sub]) and rel(out_sub, out[sub].float().cpu()) < 1e-2
 
 
+@pytest.mark.parametrize("counts", [
+    [1, 16, 17, 32, 33, 48, 64, 65],              # wave row 0 with 1, 1, 2, 2, 3, 3, 4 and 5 live blocks; wave row 1 without rows
+    [100, 128, 129, 144, 160, 161, 193, 224],     # wave row 0 full; wave row 1 with 0, 0, 1, 1, 2, 3, 5 and 6 live blocks
+    [225, 255, 256, 257, 300, 511, 513, 0],       # tiles that run the unchecked loop, tails behind full tiles, an empty group
+])
+def test_ragged_row_tiles_of_every_block_count(dev, oracle, counts):
+    """Groups whose last row tile has every number of live 16-row blocks a wave can meet: each count runs its own copy
+    of the grouped GEMMs' K loop, blocks inside a count but past the group compute on rows that were never loaded, and
+    the fused epilogues (SwiGLU with the h A2 product; SwiGLU backward with the adapter gradients' row and column sums)
+    must keep those rows out of every sum.  Pre-dispatched rows, LoRA r=16, forward and backward against the fp32 oracle."""
+    import moe_distributed_training_amd as moe
+    d, f, r, alpha = 256, 512, 16, 32.0
+    E, R = len(counts), sum(counts)
+    g = torch.Generator(device=dev).manual_seed(11)
+    rn = lambda *s, std=1.0: (torch.randn(*s, generator=g, device=dev) * std).bfloat16()
+    w1, w2, w3 = rn(E, f, d, std=0.05), rn(E, f, d, std=0.05), rn(E, f, d, std=0.05)
+    lora = {"w1": (rn(E, d, r, std=0.05), rn(E, r, f, std=0.05)), "w3": (rn(E, d, r, std=0.05), rn(E, r, f, std=0.05)),
+            "w2": (rn(E, f, r, std=0.05), rn(E, r, d, std=0.05))}
+    xr, dy = rn(R, d), rn(R, d)
+    e_of_row = torch.repeat_interleave(torch.arange(E), torch.tensor(counts))[torch.randperm(R, generator=torch.Generator().manual_seed(5))]
+    sei, ssi = oracle.flatten_and_sort(e_of_row)
+    eo = torch.bincount(sei, minlength=E).cumsum(0)
+    lt, views = _views({n: (a.cpu(), b.cpu()) for n, (a, b) in lora.items()}, dev)
+    xg = xr.clone().requires_grad_(True)
+    y = moe.fused_expert_mlp(xg, w1, w2, w3, 1, ssi.int().to(dev), eo.int().to(dev), views, alpha)
+    y.backward(dy)
+    xo = xr.float().cpu().requires_grad_(True)
+    lo = {n: (a.float().cpu().requires_grad_(True), b.float().cpu().requires_grad_(True)) for n, (a, b) in lora.items()}
+    ref, _ = oracle.moe_block(xo, None, w1.float().cpu(), w2.float().cpu(), w3.float().cpu(), 1, lo, alpha,
+                              routing=(torch.ones(R, 1), e_of_row[:, None]))
+    ref.backward(dy.float().cpu())
+    assert torch.isfinite(y.float()).all() and torch.isfinite(xg.grad.float()).all()
+    assert rel(y, ref) < 1e-2 and rel(xg.grad, xo.grad) < 1e-2
+    for n in ("w1", "w3", "w2"):
+        assert torch.isfinite(lt[n][0].grad.float()).all() and torch.isfinite(lt[n][1].grad.float()).all()
+        check_expert_grads(lt[n][0].grad, lo[n][0].grad, f"dA {n}", tol=TINY_GROUP_TOL)
+        check_expert_grads(lt[n][1].grad, lo[n][1].grad, f"dB {n}", tol=TINY_GROUP_TOL)
+
+
 @pytest.mark.slow
 def test_skewed_full_size_properties(dev, oracle):
     """BASELINE configs[3] at its full size (T=16384, E=8, top-2, Zipf-skewed routing, LoRA r=16, fwd+bwd) through
