@@ -5,6 +5,7 @@
 #include "common.h"
 #include "kernels.h"
 #include <mutex>
+#include <type_traits>
 
 namespace {
 
@@ -125,96 +126,74 @@ __global__ void router_topk_kernel(const float* __restrict__ logits, float* __re
     softmax_topk_token(logits + t * E, scores + t * E, topw + t * k, topi + t * k, E, k, renorm);
 }
 
-// Logits, softmax and top-k in one launch for up to ROUTER_EXPERT_GROUP experts whose weights fit in LDS (Mixtral:
-// 8 x 4096 bf16 = 64 KiB).  A workgroup copies the router weight to LDS once and handles 16 tokens, 2 per wave (one token per wave measured slower): the
-// activation rows stream from HBM (the only large traffic), the weight chunks come from LDS instead of being
-// re-fetched through the cache by every wave.  The accumulation order per logit is the one of router_logits_kernel
-// (lane-local chunks in ascending k, then the same butterfly), so both produce identical bits.
-constexpr int RF_WAVES = 8, RF_TOKENS_PER_WAVE = 2, RF_TOKENS = RF_WAVES * RF_TOKENS_PER_WAVE;
-constexpr int RF_BATCH = 8;   // K chunks whose activation loads are in flight together (64 lanes x 8 elements each)
+// Logits, softmax and top-k in one launch for up to ROUTER_EXPERT_GROUP experts of a 2-byte type, the logits on the
+// matrix cores.  A workgroup of 8 waves handles 16 tokens; wave w takes the w-th eighth of the hidden dimension: it
+// requests all of its operand fragments at once -- 16 bytes per lane straight from global memory in v_mfma_f32_16x16x32
+// layout (lane i + 16 g holds row i, k = 8 g .. 8 g + 7 of a 32-wide step; rows are tokens for the activations and
+// experts for the router weight, whose 64 KiB stay in L2) -- so the kernel pays one memory round trip, and then runs one
+// MFMA per step.  With the weight fragment as first operand a lane ends up with 4 experts' partial logits of one
+// token; the eight waves' partial sums meet in LDS and are added in wave order (fixed: the result does not depend on
+// timing).  The summation order differs from router_logits_kernel's, so the two agree to fp32 rounding, not bit for bit.
+constexpr int RM_WAVES = 8, RM_TOKENS = 16;
+constexpr int RM_BATCH = 16;   // 32-wide K steps whose loads are in flight together (16 steps x 8 waves = 4096 columns)
 template <typename T>
-__global__ void __launch_bounds__(RF_WAVES * 64) router_fused_kernel(const T* __restrict__ x, int64_t ldx,
-                                                                     const T* __restrict__ wg, int64_t ldw,
-                                                                     float* __restrict__ logits, float* __restrict__ scores,
-                                                                     float* __restrict__ topw, int32_t* __restrict__ topi,
-                                                                     int64_t ntok, int d, int E, int k, int renorm)
+__global__ void __launch_bounds__(RM_WAVES * 64) router_mfma_kernel(const T* __restrict__ x, int64_t ldx,
+                                                                    const T* __restrict__ wg, int64_t ldw,
+                                                                    float* __restrict__ logits, float* __restrict__ scores,
+                                                                    float* __restrict__ topw, int32_t* __restrict__ topi,
+                                                                    int64_t ntok, int d, int E, int k, int renorm)
 {
-    extern __shared__ __attribute__((aligned(16))) uint8_t rf_smem[];
-    T* s_w = (T*)rf_smem;                                        // [E][d]
-    __shared__ float s_logits[RF_TOKENS][ROUTER_EXPERT_GROUP];
+    __shared__ float s_part[RM_WAVES][RM_TOKENS][16];
+    __shared__ float s_logits[RM_TOKENS][ROUTER_EXPERT_GROUP];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int64_t t0 = (int64_t)blockIdx.x * RF_TOKENS + wave * RF_TOKENS_PER_WAVE;
-    const T* xrow[RF_TOKENS_PER_WAVE];
+    const int64_t t0 = (int64_t)blockIdx.x * RM_TOKENS;
+    const int row = lane & 15, kc = lane >> 4;
+    const int64_t tok = (t0 + row < ntok) ? t0 + row : ntok - 1;      // tokens past the end re-read the last one
+    const T* xp = x + tok * ldx + kc * 8;
+    const T* wp = wg + (int64_t)(row < E ? row : E - 1) * ldw + kc * 8;   // rows past the last expert enter as zeros
+    const int nsteps = d / 32;
+    const int s_end = nsteps * (wave + 1) / RM_WAVES;
+    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+    for (int s0 = nsteps * wave / RM_WAVES; s0 < s_end; s0 += RM_BATCH) {
+        uint4 xa[RM_BATCH], wa[RM_BATCH];
 #pragma unroll
-    for (int i = 0; i < RF_TOKENS_PER_WAVE; ++i) xrow[i] = x + ((t0 + i < ntok) ? t0 + i : ntok - 1) * ldx;
-    // The router weight goes global -> LDS with direct-to-LDS loads (64 consecutive 16-byte chunks per instruction,
-    // no registers, no wait between them), then the first batch of activation chunks is requested; one wait covers
-    // both, so the kernel pays a single memory round trip before it starts computing.  Lanes past the last chunk of
-    // a partial group re-read the last chunk into the padding behind the image.
-    const int chunks_per_row = d / 8;                            // 16-byte chunks (2-byte elements)
-    const int nchunks = E * chunks_per_row;
-    const uint32_t lds_w = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)LDS_PTR(s_w));
-    for (int c0 = wave * 64; c0 < nchunks; c0 += RF_WAVES * 64) {
-        const int c = (c0 + lane < nchunks) ? c0 + lane : nchunks - 1;
-        const T* src = wg + (int64_t)(c / chunks_per_row) * ldw + (c % chunks_per_row) * 8;
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(__builtin_amdgcn_readfirstlane(lds_w + (uint32_t)c0 * 16)), "v"(src) : "memory", "m0");
-    }
-    uint4 xr[RF_BATCH][RF_TOKENS_PER_WAVE];
-    auto request = [&](int kbase) {
-#pragma unroll
-        for (int c = 0; c < RF_BATCH; ++c) {
-            const int k0 = kbase + c * 512 + lane * 8;
-#pragma unroll
-            for (int i = 0; i < RF_TOKENS_PER_WAVE; ++i) xr[c][i] = (k0 < d) ? *(const uint4*)(xrow[i] + k0) : make_uint4(0, 0, 0, 0);
+        for (int i = 0; i < RM_BATCH; ++i) {
+            const int st = (s0 + i < s_end) ? s0 + i : s_end - 1;
+            xa[i] = *(const uint4*)(xp + (int64_t)st * 32);
+            wa[i] = *(const uint4*)(wp + (int64_t)st * 32);
         }
-    };
-    request(0);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wave's share of the weight image has landed (and its activations)
-    __syncthreads();
-    float acc[RF_TOKENS_PER_WAVE][ROUTER_EXPERT_GROUP];
 #pragma unroll
-    for (int i = 0; i < RF_TOKENS_PER_WAVE; ++i)
-#pragma unroll
-        for (int j = 0; j < ROUTER_EXPERT_GROUP; ++j) acc[i][j] = 0.f;
-    for (int kbase = 0; kbase < d; kbase += RF_BATCH * 512) {
-        if (kbase > 0) request(kbase);
-#pragma unroll
-        for (int c = 0; c < RF_BATCH; ++c) {
-            const int k0 = kbase + c * 512 + lane * 8;
-            if (k0 < d) {
-                float xv[RF_TOKENS_PER_WAVE][8];
-#pragma unroll
-                for (int i = 0; i < RF_TOKENS_PER_WAVE; ++i) {
-                    const T* e8 = (const T*)&xr[c][i];
-#pragma unroll
-                    for (int u = 0; u < 8; ++u) xv[i][u] = Elem<T>::ld(e8 + u);
-                }
-#pragma unroll
-                for (int j = 0; j < ROUTER_EXPERT_GROUP; ++j) {
-                    const int e = (j < E) ? j : E - 1;
-                    float wv[8];
-                    load8<T>(s_w + (int64_t)e * d + k0, wv, 8, true);
-#pragma unroll
-                    for (int i = 0; i < RF_TOKENS_PER_WAVE; ++i)
-#pragma unroll
-                        for (int u = 0; u < 8; ++u) acc[i][j] = fmaf(xv[i][u], wv[u], acc[i][j]);
+        for (int i = 0; i < RM_BATCH; ++i) {
+            if (s0 + i < s_end) {
+                uint4 w4 = wa[i];
+                if (row >= E) w4 = make_uint4(0, 0, 0, 0);
+                if constexpr (sizeof(T) == 2 && std::is_same<T, __hip_bfloat16>::value) {
+                    union { uint4 u; bf16x8_t v; } a, b;
+                    a.u = w4; b.u = xa[i];
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, acc, 0, 0, 0);
+                } else {
+                    typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+                    union { uint4 u; f16x8_t v; } a, b;
+                    a.u = w4; b.u = xa[i];
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a.v, b.v, acc, 0, 0, 0);
                 }
             }
         }
     }
-#pragma unroll
-    for (int i = 0; i < RF_TOKENS_PER_WAVE; ++i)
-#pragma unroll
-        for (int j = 0; j < ROUTER_EXPERT_GROUP; ++j) {
-            const float sum = wave_sum(acc[i][j]);
-            if (lane == 0 && j < E) {
-                s_logits[wave * RF_TOKENS_PER_WAVE + i][j] = sum;
-                if (t0 + i < ntok) logits[(t0 + i) * E + j] = sum;
-            }
-        }
+    // acc[r] = partial logit of token `row`, expert 4 * kc + r
+    *(f32x4_t*)&s_part[wave][row][4 * kc] = acc;
     __syncthreads();
-    const int64_t t = (int64_t)blockIdx.x * RF_TOKENS + tid;
-    if (tid < RF_TOKENS && t < ntok) softmax_topk_token(s_logits[tid], scores + t * E, topw + t * k, topi + t * k, E, k, renorm);
+    if (tid < RM_TOKENS * ROUTER_EXPERT_GROUP) {
+        const int t = tid / ROUTER_EXPERT_GROUP, e = tid % ROUTER_EXPERT_GROUP;
+        float sum = s_part[0][t][e];
+#pragma unroll
+        for (int w = 1; w < RM_WAVES; ++w) sum += s_part[w][t][e];
+        s_logits[t][e] = sum;
+        if (e < E && t0 + t < ntok) logits[(t0 + t) * E + e] = sum;
+    }
+    __syncthreads();
+    const int64_t t = t0 + tid;
+    if (tid < RM_TOKENS && t < ntok) softmax_topk_token(s_logits[tid], scores + t * E, topw + t * k, topi + t * k, E, k, renorm);
 }
 
 // Backward of softmax -> top-k -> renormalise with respect to the logits.
@@ -375,6 +354,128 @@ __global__ void __launch_bounds__(SORT_THREADS) sort_scatter_kernel(const void* 
     }
 }
 
+// The whole sort in one launch, for batches small enough that every workgroup can afford to read ALL assignment ids
+// itself: a workgroup counts, per expert, the entries before its own chunk and the entries altogether (LDS atomics, each
+// wave into its own rows), which gives it its chunk's destination bases without a histogram
+// launch and a scan launch before it; then it scatters its chunk exactly as sort_scatter_kernel does.  Workgroup 0 also
+// writes the per-expert counts, the inclusive offsets and the block table.  Same results as the three-launch path.
+constexpr int64_t SORT_ONE_LAUNCH_MAX_ROWS = 16384;
+constexpr int SORT_ONE_LAUNCH_MAX_EXPERTS = 256;
+static_assert(SORT_CHUNK % 64 == 0, "a 64-entry group of the counting pass lies wholly before a chunk or not at all");
+__global__ void __launch_bounds__(SORT_THREADS) sort_one_launch_kernel(const void* __restrict__ expert_idx, int in64,
+                                                                       int64_t R, int E, int block_m,
+                                                                       void* __restrict__ sorted_expert,
+                                                                       void* __restrict__ sorted_pos, int out64,
+                                                                       void* __restrict__ counts, void* __restrict__ offsets,
+                                                                       void* __restrict__ padded_blocks, int64_t padded_cap,
+                                                                       int32_t* __restrict__ num_padded, int32_t* __restrict__ inv)
+{
+    extern __shared__ int32_t sh[];  // before[NW][E], total[NW][E], then cursor[NW][E]
+    constexpr int NW = SORT_THREADS / 64;
+    constexpr int PER_WAVE = SORT_CHUNK / NW;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    int32_t* before = sh;
+    int32_t* total = sh + NW * E;
+    int32_t* cur = sh + 2 * NW * E;
+    for (int i = threadIdx.x; i < 3 * NW * E; i += SORT_THREADS) sh[i] = 0;
+    __syncthreads();
+    const int64_t chunk_base = (int64_t)blockIdx.x * SORT_CHUNK;
+    // counts over the whole array: wave w walks entries [64 (w + NW j), +64), sixteen groups' ids requested together;
+    // LDS atomics into the wave's own rows (integer counts: the order of the additions does not matter)
+    constexpr int SB = 16;
+    for (int64_t p0 = (int64_t)w * 64; p0 < R; p0 += (int64_t)NW * 64 * SB) {
+        int ev[SB];
+        int64_t raw[SB];
+        // (one branch on the index width around all the loads, so that they are in flight together; entries past the
+        // end re-read the last one and are dropped below)
+        if (in64) {
+#pragma unroll
+            for (int j = 0; j < SB; ++j) { const int64_t p = p0 + (int64_t)j * NW * 64 + lane; raw[j] = ((const int64_t*)expert_idx)[p < R ? p : R - 1]; }
+        } else {
+#pragma unroll
+            for (int j = 0; j < SB; ++j) { const int64_t p = p0 + (int64_t)j * NW * 64 + lane; raw[j] = ((const int32_t*)expert_idx)[p < R ? p : R - 1]; }
+        }
+#pragma unroll
+        for (int j = 0; j < SB; ++j) {
+            const int64_t p = p0 + (int64_t)j * NW * 64 + lane;
+            ev[j] = (p < R && raw[j] >= 0 && raw[j] < E) ? (int)raw[j] : -1;
+        }
+#pragma unroll
+        for (int j = 0; j < SB; ++j) {
+            if (ev[j] >= 0) {
+                atomicAdd(&total[w * E + ev[j]], 1);
+                // a 64-entry group lies wholly before the chunk or not at all (chunks are multiples of 64 entries)
+                if (p0 + (int64_t)j * NW * 64 < chunk_base) atomicAdd(&before[w * E + ev[j]], 1);
+            }
+        }
+    }
+    // per-wave histogram of the own chunk (as in sort_scatter_kernel)
+    const int64_t wbase = chunk_base + (int64_t)w * PER_WAVE;
+    for (int i = lane; i < PER_WAVE; i += 64) {
+        const int64_t p = wbase + i;
+        if (p < R) {
+            const int64_t e = load_idx(expert_idx, p, in64);
+            if (e >= 0 && e < E) atomicAdd(&cur[w * E + (int)e], 1);
+        }
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < E; e += SORT_THREADS) {
+        int32_t b = 0, t = 0;
+        for (int ww = 0; ww < NW; ++ww) { b += before[ww * E + e]; t += total[ww * E + e]; }
+        before[e] = b;
+        total[e] = t;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        // exclusive scan over the experts; workgroup 0 publishes counts, offsets and the block table
+        const bool pub = blockIdx.x == 0;
+        int64_t run = 0, nb = 0;
+        for (int e = 0; e < E; ++e) {
+            const int64_t c = total[e];
+            const int64_t start = run;
+            run += c;
+            if (pub) {
+                if (counts) store_idx(counts, e, c, out64);
+                if (offsets) store_idx(offsets, e, run, out64);
+                if (padded_blocks)
+                    for (int64_t s_ = start; s_ < run; s_ += block_m) { if (nb < padded_cap) store_idx(padded_blocks, nb, s_, out64); ++nb; }
+            }
+            total[e] = (int32_t)start;
+        }
+        if (pub && num_padded) *num_padded = (int32_t)nb;
+    }
+    __syncthreads();
+    // exclusive prefix over waves, seeded with this chunk's base = the expert's start + its entries before the chunk
+    for (int e = threadIdx.x; e < E; e += SORT_THREADS) {
+        int32_t run = total[e] + before[e];
+        for (int ww = 0; ww < NW; ++ww) { const int32_t c = cur[ww * E + e]; cur[ww * E + e] = run; run += c; }
+    }
+    __syncthreads();
+    volatile int32_t* cursor = cur + w * E;
+    for (int i0 = 0; i0 < PER_WAVE; i0 += 64) {
+        const int64_t p = wbase + i0 + lane;
+        int e = -1;
+        if (p < R) { const int64_t ee = load_idx(expert_idx, p, in64); e = (ee >= 0 && ee < E) ? (int)ee : -1; }
+        uint64_t rem = __ballot(e >= 0);
+        while (rem) {
+            const int leader = __ffsll((unsigned long long)rem) - 1;
+            const int e0 = __shfl(e, leader, 64);
+            const uint64_t m = __ballot(e == e0);
+            if (e == e0) {
+                const int rank = __popcll(m & ((1ull << lane) - 1ull));
+                const int32_t dst = cursor[e0] + rank;
+                store_idx(sorted_expert, dst, e0, out64);
+                store_idx(sorted_pos, dst, p, out64);
+                if (inv) inv[p] = dst;
+            }
+            __builtin_amdgcn_wave_barrier();
+            if (lane == leader) cursor[e0] += __popcll(m);
+            __builtin_amdgcn_wave_barrier();
+            rem &= ~m;
+        }
+    }
+}
+
 // offsets[e] = number of entries of the non-decreasing array sorted_expert that are <= e  (inclusive running count)
 __global__ void offsets_from_sorted_kernel(const void* __restrict__ sorted_expert, int in64, int64_t R, int E,
                                            void* __restrict__ offsets, int out64)
@@ -424,28 +525,19 @@ int moe_launch_router_forward(const void* x, int64_t ldx, const void* wg, int64_
                               int renorm, hipStream_t stream)
 {
     if (ntok == 0) return MOE_OK;
-    const size_t wbytes = (size_t)E * (size_t)d * 2;
-    const bool fused = dtype != MOE_F32 && E <= ROUTER_EXPERT_GROUP && wbytes <= 64 * 1024 && d % 8 == 0 && d < (1 << 30) &&
+    const bool fused = dtype != MOE_F32 && E <= ROUTER_EXPERT_GROUP && d % 32 == 0 && d >= 32 && d < (1 << 30) &&
                        ((uintptr_t)x % 16 == 0) && ((uintptr_t)wg % 16 == 0) && ldx % 8 == 0 && ldw % 8 == 0;
     if (!fused) {
         const int rc = moe_launch_router_logits(x, ldx, wg, ldw, dtype, logits, ntok, d, E, stream);
         return rc != MOE_OK ? rc : moe_launch_router_topk(logits, scores, topw, topi, ntok, E, k, renorm, stream);
     }
-    const unsigned grid = (unsigned)((ntok + RF_TOKENS - 1) / RF_TOKENS);
-    const size_t lds_bytes = (wbytes + 1023) / 1024 * 1024;   // whole 64-chunk groups
-    if (dtype == MOE_BF16) {
-        static std::atomic<bool> attr_set{false};   // forward and backward may call from different host threads
-        auto kern = router_fused_kernel<__hip_bfloat16>;
-        if (!attr_set) { if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024) != hipSuccess) return MOE_ERR_LAUNCH; attr_set = true; }
-        hipLaunchKernelGGL(kern, dim3(grid), dim3(RF_WAVES * 64), lds_bytes, stream, (const __hip_bfloat16*)x, ldx, (const __hip_bfloat16*)wg, ldw,
-                           logits, scores, topw, topi, ntok, (int)d, E, k, renorm);
-    } else {
-        static std::atomic<bool> attr_set{false};   // forward and backward may call from different host threads
-        auto kern = router_fused_kernel<__half>;
-        if (!attr_set) { if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024) != hipSuccess) return MOE_ERR_LAUNCH; attr_set = true; }
-        hipLaunchKernelGGL(kern, dim3(grid), dim3(RF_WAVES * 64), lds_bytes, stream, (const __half*)x, ldx, (const __half*)wg, ldw,
-                           logits, scores, topw, topi, ntok, (int)d, E, k, renorm);
-    }
+    const unsigned grid = (unsigned)((ntok + RM_TOKENS - 1) / RM_TOKENS);
+    if (dtype == MOE_BF16)
+        hipLaunchKernelGGL(router_mfma_kernel<__hip_bfloat16>, dim3(grid), dim3(RM_WAVES * 64), 0, stream, (const __hip_bfloat16*)x, ldx,
+                           (const __hip_bfloat16*)wg, ldw, logits, scores, topw, topi, ntok, (int)d, E, k, renorm);
+    else
+        hipLaunchKernelGGL(router_mfma_kernel<__half>, dim3(grid), dim3(RM_WAVES * 64), 0, stream, (const __half*)x, ldx,
+                           (const __half*)wg, ldw, logits, scores, topw, topi, ntok, (int)d, E, k, renorm);
     return moe_launch_status();
 }
 
@@ -480,6 +572,12 @@ int moe_launch_sort(const void* expert_idx, int in64, int64_t R, int E, int bloc
     if (E < 1 || E > 4096 || R < 0 || block_m < 1) return MOE_ERR_BAD_ARG;
     if (workspace_bytes < moe_sort_ws_bytes(R, E)) return MOE_ERR_WORKSPACE;
     const int nblk = (int)((R + SORT_CHUNK - 1) / SORT_CHUNK);
+    if (nblk > 0 && R <= SORT_ONE_LAUNCH_MAX_ROWS && E <= SORT_ONE_LAUNCH_MAX_EXPERTS) {
+        hipLaunchKernelGGL(sort_one_launch_kernel, dim3(nblk), dim3(SORT_THREADS), 3 * (SORT_THREADS / 64) * E * sizeof(int32_t), stream,
+                           expert_idx, in64, R, E, block_m, sorted_expert, sorted_pos, out64, counts, offsets, padded_blocks,
+                           padded_cap, num_padded, inv);
+        return moe_launch_status();
+    }
     int32_t* hist = (int32_t*)workspace;
     if (nblk > 0)
         hipLaunchKernelGGL(sort_hist_kernel, dim3(nblk), dim3(SORT_THREADS), E * sizeof(int32_t), stream, expert_idx,

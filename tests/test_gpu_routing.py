@@ -57,10 +57,16 @@ def test_router_end_to_end(dev, oracle, dtype, T, d, E):
     assert margin > 1e-6, "test data has a near tie; pick another seed"
     assert torch.equal(idx.cpu(), io)
     assert torch.allclose(w.cpu(), wo, atol=1e-5)
-    # the one-call form (one fused launch for <= 8 experts of a 2-byte type, two launches otherwise) gives the same bits
+    # the one-call form: two launches give the same bits as the two calls; the single fused launch (<= 8 experts of a
+    # 2-byte type, hidden size a multiple of 32) sums its logits on the matrix cores in another order -- fp32 rounding
+    # apart, the same indices, and exactly the softmax / top-k of ITS logits
     l2, s2, w2, i2 = router.router_forward(x.to(dev), wg.to(dev), k)
-    s1, w1, i1 = router.router_topk(logits, k)
-    assert torch.equal(l2, logits) and torch.equal(s2, s1) and torch.equal(w2, w1) and torch.equal(i2, i1)
+    s1, w1, i1 = router.router_topk(l2, k)
+    assert torch.equal(s2, s1) and torch.equal(w2, w1) and torch.equal(i2, i1)
+    if dtype == torch.float32 or E > 8 or d % 32 != 0:
+        assert torch.equal(l2, logits)
+    else:
+        assert torch.allclose(l2.cpu(), lo, atol=2e-5, rtol=1e-5) and torch.equal(i2.cpu().long(), io)
 
 
 def test_router_forward_ragged_token_count(dev, oracle):
