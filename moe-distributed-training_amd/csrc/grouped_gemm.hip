@@ -461,12 +461,13 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
         int bs = 0;   // B stage of tile kt
         // A tail tile of at most two row blocks has next to no MFMA work and would run through K several times faster than
         // the full row tiles that share its weight tiles: the weight tiles it fetches are then gone from L2 again before
-        // those arrive, and its requests compete with theirs.  Its waves therefore take at least PACE_CYCLES per K tile (a
-        // full tile cannot take less: 2048 cycles are its MFMAs alone), which keeps it just ahead of them -- close enough
-        // to act as their prefetcher.  Measured over eight routing draws of 8192 rows: the GEMM launches other than the
-        // gate/up pair 1-2 % faster; the pair launch, with sixteen rounds of tiles, is bound by the sum of its tiles' times
-        // and runs slower with paced tails, so it is left alone.
-        constexpr bool PACED = !FULL && NBLK <= 2 && !(EPI_IS_PAIR(EPI));
+        // those arrive (measured on the gate/up launch: 0.8 GB more fetched from memory with three such tails), and its
+        // requests compete with theirs.  Its waves therefore take at least PACE_CYCLES per K tile (a full tile cannot
+        // take less: 2048 cycles are its MFMAs alone), which keeps it just ahead of them -- close enough to act as their
+        // prefetcher.  Measured over eight routing draws of 8192 rows: the launches of few rounds 1-2 % faster; the gate/up
+        // launch, whose sixteen rounds are bound by the sum of the tiles' times, 2 % slower than with unpaced tails --
+        // the price of not fetching those weight tiles twice.
+        constexpr bool PACED = !FULL && NBLK <= 2;
         constexpr int64_t PACE_CYCLES = 2048;
         int64_t pace_t0 = PACED ? (int64_t)__builtin_readcyclecounter() : 0;
         // one K tile; SLAB: the activation loads it requests (for tile kt+2) fetch the slab image instead
