@@ -81,6 +81,26 @@ def test_router_forward_ragged_token_count(dev, oracle):
         assert torch.allclose(s.cpu(), so, atol=1e-6) and torch.allclose(w.cpu(), wo, atol=1e-5)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,d,E,k", [(5, 32, 1, 1), (40, 96, 3, 2), (100, 544, 8, 2), (16, 8192, 8, 8), (1000, 1024, 7, 3)])
+def test_router_matrix_core_kernel_shapes(dev, oracle, dtype, T, d, E, k):
+    """The one-launch router (logits on the matrix cores) at hidden sizes that leave some of its eight waves without a
+    K step (32, 96), that split unevenly over them (544 = 17 steps), with fewer than 8 experts (the unused rows of the
+    weight operand must enter as zeros) and with token counts that do not fill its 16-token workgroups."""
+    _, router, _ = _mods()
+    torch.manual_seed(T + d + E)
+    x = torch.randn(T, d).to(dtype)
+    wg = (torch.randn(E, d) * 0.05).to(dtype)
+    l, s, w, i = router.router_forward(x.to(dev), wg.to(dev), k)
+    lo, so, wo, io = oracle.router(x, wg, k)
+    srt = torch.sort(so, dim=-1, descending=True).values
+    if E > k:
+        assert (srt[:, k - 1] - srt[:, k]).abs().min() > 1e-6, "test data has a near tie; pick another seed"
+    assert torch.allclose(l.cpu(), lo, atol=3e-5, rtol=1e-5)
+    assert torch.equal(i.cpu().long(), io)
+    assert torch.allclose(s.cpu(), so, atol=1e-6) and torch.allclose(w.cpu(), wo, atol=1e-5)
+
+
 def test_reference_known_answers_on_the_device(dev):
     """The vectors the reference's own test holds (tests/test_scattermoe.py:84-85) and its documented block-table
     example (scattermoe_utils/kernels/ops.py:45-49), from the committed fixture, through the HIP path."""
