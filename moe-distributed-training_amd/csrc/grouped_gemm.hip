@@ -356,8 +356,9 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
     // number of 16-row MFMA blocks of this wave that hold at least one real row
     int mb_cnt = (nrows - wm * WTM + 15) / 16;
     mb_cnt = mb_cnt < 0 ? 0 : (mb_cnt > MB ? MB : mb_cnt);
-    // the same in every lane: as a scalar, the checks around the MFMAs of a ragged tile are scalar branches (under a
-    // vector condition the compiler masks single MFMAs instead of branching around them, and the matrix cores ignore the mask)
+    // the same in every lane: as a scalar it selects the wave's copy of the K loop with one branch, and the checks in
+    // the slab step are scalar branches (under a vector condition the compiler masks single MFMAs instead of branching
+    // around them, and the matrix cores ignore the mask)
     mb_cnt = __builtin_amdgcn_readfirstlane(mb_cnt);
 
     const int kb = ktiles * part / nparts;
@@ -367,8 +368,8 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
     // One direct-to-LDS load instruction of a K tile's activation (issue_a) or weight (issue_b) image, into the given
     // stage.  K tiles past the end re-read the last one (into the stage such a tile would use, which nobody reads any
     // more), which keeps the main loop free of branches around the loads.  Activation instructions whose 8 rows lie
-    // past the tile's last 32-row block are dropped when `ragged` is set (the MFMAs that would read them are skipped
-    // too); the wait counts of the main loop only ever leave weight instructions in flight, which are never dropped,
+    // past the tile's last 32-row block are dropped when `ragged` is set (what MFMAs compute from such rows is never
+    // stored or summed); the wait counts of the main loop only ever leave weight instructions in flight, which are never dropped,
     // so they do not depend on how many activation instructions were.
     const int live_rows = (nrows + 31) / 32 * 32;
     auto issue_a = [&](int kt, int jj, int stage, bool ragged) {
