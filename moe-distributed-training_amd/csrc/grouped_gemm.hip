@@ -486,8 +486,8 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
                 // ra / rb: where the fragments of the next half step come from; for the last one of a tile, the first of
                 // the next tile.  (After the last tile this fetches fragments nobody uses.)
                 if (hs == 3) {
-                    if (PACED) {   // (see PACE_CYCLES)
-                        while ((int64_t)__builtin_readcyclecounter() - pace_t0 < PACE_CYCLES) __builtin_amdgcn_s_sleep(2);
+                    if (PACED) {   // (see PACE_CYCLES; a sleep is 128 cycles, so the count bounds the wait whatever the counter's rate)
+                        for (int n = 0; n < 24 && (int64_t)__builtin_readcyclecounter() - pace_t0 < PACE_CYCLES; ++n) __builtin_amdgcn_s_sleep(2);
                         pace_t0 = (int64_t)__builtin_readcyclecounter();
                     }
                     __builtin_amdgcn_s_waitcnt(0x0F70 | LPT);   // all but the youngest LPT loads: tile kt+1 has landed
