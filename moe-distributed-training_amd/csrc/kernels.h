@@ -175,8 +175,6 @@ int moe_launch_combine_fwd(const void* y, int64_t ldy, void* out, int64_t ldo, c
                            hipStream_t stream);
 int moe_launch_combine_dgates(const void* y, int64_t ldy, const void* dout, int64_t ldd, void* dgates, int gdtype,
                               const int32_t* inv, int k, int64_t ntok, int64_t ncols, int dtype, hipStream_t stream);
-int moe_launch_copy_rows_bf16(const void* src, int64_t lds_, void* dst, int64_t ldd, int64_t rows, int64_t cols,
-                              hipStream_t stream);
 int moe_launch_swiglu_fwd(const void* g, const void* u, void* h, int64_t n, int dtype, hipStream_t stream);
 int moe_launch_swiglu_bwd(const void* g, const void* u, const void* dh, void* dg, void* du, int64_t n, int dtype,
                           hipStream_t stream);

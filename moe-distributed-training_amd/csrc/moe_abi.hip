@@ -429,12 +429,10 @@ static inline size_t sk_bytes_mlp(int64_t R, int E, int64_t d, int64_t f)
 }
 // column-tile partials of the two fused column contractions of the dh GEMM: [2][ceil(f / 256)][R][16] fp32
 static inline size_t cc_bytes(int64_t R, int64_t f) { return (size_t)2 * (size_t)((f + 255) / 256) * (size_t)R * 16 * sizeof(float); }
-static inline bool bad_pitch(int64_t ld) { return (ld * 2) % 4096 == 0; }
-static inline size_t repitch_bytes(int64_t R, int64_t d) { return al((size_t)R * (size_t)(d + 64) * 2); }
 
 size_t moe_mlp_workspace_bytes(int64_t R, int E, int64_t d, int64_t f, int rank)
 {
-    size_t n = repitch_bytes(R, d) + al(sk_bytes_mlp(R, E, d, f)) + 256;
+    size_t n = al(sk_bytes_mlp(R, E, d, f)) + 256;
     if (rank <= 0) return n;
     const int64_t mx = d > f ? d : f;
     const size_t C = (size_t)(rank + 15) / 16;   // 16-wide chunks per adapter
@@ -467,7 +465,7 @@ int moe_mlp_fwd(const void* x, int64_t ldx, const void* w1, const void* w3, cons
     const bool has_lora = lora && lora[0];
     if (has_lora && (!ls || !saved || rank < 1)) return MOE_ERR_BAD_ARG;
     if (!mlp_shapes_ok(d, f, ldx, has_lora ? rank : 0, w1, w3, w2, x)) return MOE_ERR_UNSUPPORTED;
-    if (!mlp_sizes_ok(R / fan_out, bad_pitch(ldx) ? d + 64 : ldx, d, f)) return MOE_ERR_UNSUPPORTED;
+    if (!mlp_sizes_ok(R / fan_out, ldx, d, f)) return MOE_ERR_UNSUPPORTED;
     if (R == 0) return MOE_OK;
     hipStream_t st = S(stream);
     uint8_t* sv = (uint8_t*)saved;
@@ -477,14 +475,6 @@ int moe_mlp_fwd(const void* x, int64_t ldx, const void* w1, const void* w3, cons
     Bump ws(workspace, workspace_bytes);
     void* skws = ws.take(sk_bytes_mlp(R, E, d, f));
     bool counters_clean = has_lora;   // K-split counters: zeroed by the adapter pack launch; a GEMM launch that uses them leaves them zero
-    const void* xg = x;          // A operand of the w1/w3 GEMM
-    int64_t ldxg = ldx;
-    if (bad_pitch(ldx)) {
-        TIMED("fwd.repitch_x");
-        void* xp = ws.take(repitch_bytes(R / fan_out, d));
-        TRY(moe_launch_copy_rows_bf16(x, ldx, xp, d + 64, R / fan_out, d, st));
-        xg = xp; ldxg = d + 64;
-    }
     // An adapter of rank r is worked through as C = ceil(r / 16) independent 16-wide chunks of its rank columns:
     // x A B = sum_c (x A[:, c]) B[c, :].  saved: per chunk c, Q1, Q3, Q2, Qt1, Qt3, Qt2 (six q_bytes blocks).
     const int C = has_lora ? (rank + 15) / 16 : 0;
@@ -525,7 +515,7 @@ int moe_mlp_fwd(const void* x, int64_t ldx, const void* w1, const void* w3, cons
     }
     {
         MoeGemmParams p = {};
-        p.X[0] = (const uint16_t*)xg; p.ldx = ldxg; p.nseg = 1;
+        p.X[0] = (const uint16_t*)x; p.ldx = ldx; p.nseg = 1;
         p.W[0] = (const uint16_t*)w1; p.W[1] = (const uint16_t*)w3; p.swe = f * d; p.ldw = d; p.nn = 0;
         if (has_lora) {   // gate slabs first, then up slabs
             for (int c = 0; c < C; ++c) {
@@ -589,7 +579,7 @@ int moe_mlp_bwd(const void* dy, int64_t lddy, int dy_grouped, int dy_fan_out, co
     if (!mlp_shapes_ok(d, f, ldx, has_lora ? rank : 0, w1, w3, w2, x) || lddy % 8 != 0 || !aligned16(dy))
         return MOE_ERR_UNSUPPORTED;
     if (dy_fan_out < 1 || fan_out < 1) return MOE_ERR_BAD_ARG;
-    if (!mlp_sizes_ok(dy_grouped ? 256 : R / dy_fan_out, bad_pitch(lddy) ? d + 64 : lddy, d, f)) return MOE_ERR_UNSUPPORTED;
+    if (!mlp_sizes_ok(dy_grouped ? 256 : R / dy_fan_out, lddy, d, f)) return MOE_ERR_UNSUPPORTED;
     hipStream_t st = S(stream);
     const size_t qb = q_bytes(R);
     const int64_t ldt = pad_rows(R);
@@ -612,15 +602,6 @@ int moe_mlp_bwd(const void* dy, int64_t lddy, int dy_grouped, int dy_fan_out, co
     Bump ws(workspace, workspace_bytes);
     void* skws = ws.take(sk_bytes_mlp(R, E, d, f));
     bool counters_clean = has_lora;   // K-split counters: zeroed by the adapter pack launch; a GEMM launch that uses them leaves them zero
-    const void* dyg = dy;        // A operand of the w2-backward GEMM
-    int64_t lddyg = lddy;
-    if (bad_pitch(lddy) && R > 0) {
-        TIMED("bwd.repitch_dy");
-        const int64_t rows = dy_grouped ? R : R / dy_fan_out;
-        void* dp = ws.take(repitch_bytes(rows, d));
-        TRY(moe_launch_copy_rows_bf16(dy, lddy, dp, d + 64, rows, d, st));
-        dyg = dp; lddyg = d + 64;
-    }
     if (has_lora) {
         pq = (uint8_t*)ws.take((size_t)C * 6 * qb);
         if (fuse_rc) p2s = ws.take(qb);   // P2 times the row scale, row-major (the fused contraction's operand)
@@ -663,7 +644,7 @@ int moe_mlp_bwd(const void* dy, int64_t lddy, int dy_grouped, int dy_fan_out, co
     }
     {
         MoeGemmParams p = {};
-        p.X[0] = (const uint16_t*)dyg; p.ldx = lddyg; p.nseg = 1;
+        p.X[0] = (const uint16_t*)dy; p.ldx = lddy; p.nseg = 1;
         p.W[0] = (const uint16_t*)w2; p.swe = f * d; p.ldw = d; p.nn = 0;  // (E, K=d, N=f): n rows, k contiguous
         if (has_lora) {
             for (int c = 0; c < C; ++c) { p.Q[c] = (const uint16_t*)pqp(0, c); p.LB[c] = (const uint16_t*)la2[c]; }

@@ -171,14 +171,6 @@ __global__ void __launch_bounds__(ROW_THREADS) swiglu_bwd_kernel(const T* __rest
     Elem<T>::st(du + i, d * gv * sg);
 }
 
-// dst[r][0:cols] = src[r][0:cols] for 16-byte aligned rows (re-pitching copy; cols in 16-byte units)
-__global__ void __launch_bounds__(ROW_THREADS) copy_rows16_kernel(const uint4* __restrict__ src, int64_t lds16,
-                                                                  uint4* __restrict__ dst, int64_t ldd16, int64_t cols16)
-{
-    const int64_t r = blockIdx.x;
-    for (int64_t c = threadIdx.x; c < cols16; c += ROW_THREADS) dst[r * ldd16 + c] = src[r * lds16 + c];
-}
-
 // Router weight gradient dWg[e][c] = sum_t dlogits[t][e] * x[t][c], fp32 coefficients (no rounding of dlogits), fp32
 // accumulate.  Pass 1: workgroup (chunk, column block) sums its WG_TOKENS tokens for every expert, a thread owning N
 // consecutive columns (one 16-byte load per token) and EG experts at a time; partial[chunk][e][c] fp32.  Pass 2 adds the
@@ -303,16 +295,6 @@ int moe_launch_swiglu_bwd(const void* g, const void* u, const void* dh, void* dg
     MOE_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((swiglu_bwd_kernel<T>), dim3((unsigned)((n + ROW_THREADS - 1) / ROW_THREADS)),
                                                  dim3(ROW_THREADS), 0, stream, (const T*)g, (const T*)u, (const T*)dh,
                                                  (T*)dg, (T*)du, n));
-    return moe_launch_status();
-}
-
-int moe_launch_copy_rows_bf16(const void* src, int64_t lds_, void* dst, int64_t ldd, int64_t rows, int64_t cols,
-                              hipStream_t stream)
-{
-    if (rows == 0 || cols == 0) return MOE_OK;
-    if (cols % 8 || lds_ % 8 || ldd % 8 || ((uintptr_t)src % 16) || ((uintptr_t)dst % 16)) return MOE_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL(copy_rows16_kernel, dim3((unsigned)rows), dim3(ROW_THREADS), 0, stream, (const uint4*)src, lds_ / 8,
-                       (uint4*)dst, ldd / 8, cols / 8);
     return moe_launch_status();
 }
 
