@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define MOE_HIP_ABI_VERSION 1
+#define MOE_HIP_ABI_VERSION 2   /* 2: router weight gradient, static-scratch sort, stage-timer selection, moe_combine with k = 0; fp16 on the matrix cores (dtype argument of moe_mlp_fwd / moe_mlp_bwd) */
 
 #define MOE_OK 0
 #define MOE_ERR_BAD_ARG (-1)      /* inconsistent sizes / null pointers */
@@ -64,6 +64,9 @@ int moe_profile_get(int i, char* name, int name_cap, float* ms);
  * row, one-past-last row, K part, K parts, exchange slot, split-tile counter.  Tests use it to check that every tile
  * is covered exactly once for any group sizes. */
 int64_t moe_gemm_debug_plan_blocks(int64_t R, int E, int64_t N, int pair);
+/* number of matrix-core grouped GEMM launches this process has enqueued so far (any entry point): tests read it before
+ * and after a call to tell that a shape ran on the matrix cores and not on the generic fallback kernels */
+int64_t moe_gemm_debug_launch_count(void);
 int moe_gemm_debug_plan(const void* offsets, int off64, int E, int64_t R, int64_t K, int64_t N, int pair, int nseg,
                         int32_t* out, void* stream);
 
@@ -76,8 +79,9 @@ int moe_router_logits(const void* x, int64_t ldx, const void* wg, int64_t ldw, i
 int moe_router_topk(const float* logits, float* scores, float* topw, int32_t* topi, int64_t ntok, int E, int k,
                     int renorm, void* stream);
 /* both of the above in one call (config_utils.py:262-270): logits (T,E), scores (T,E), topw (T,k), topi (T,k); a single
- * launch when the router weight is a 2-byte type of at most 8 experts and 64 KiB (it is then held in LDS), with logits
- * bit-identical to moe_router_logits. */
+ * launch when x and the router weight are a 2-byte type, E <= 8 and d is a multiple of 32 (logits on the matrix cores,
+ * eight partial sums per logit added in a fixed order: the same top-k indices as moe_router_logits + moe_router_topk,
+ * logits equal to theirs up to fp32 rounding, not bit for bit), the two kernels of those entry points otherwise. */
 int moe_router_forward(const void* x, int64_t ldx, const void* wg, int64_t ldw, int dtype, float* logits, float* scores,
                        float* topw, int32_t* topi, int64_t ntok, int64_t d, int E, int k, int renorm, void* stream);
 /* gradient of moe_router_topk with respect to the logits given d(topw); the reference obtains it from autograd. */
@@ -99,7 +103,10 @@ int moe_router_weight_grad(const void* x, int64_t ldx, const float* dlogits, voi
  *   sorted_expert[i], sorted_pos[i]  stable ascending sort by expert id (width chosen by out64)
  *   counts[e], offsets[e]            histogram and inclusive running sum (same width)
  *   padded_blocks[0..*num_padded)    block starts, block_m rows per block, blocks never straddle experts
- *   inv[p] (int32)                   position of flat assignment p in the sorted order */
+ *   inv[p] (int32)                   position of flat assignment p in the sorted order
+ * 1 <= E <= 4096, else MOE_ERR_BAD_ARG before anything is enqueued.  Ids outside [0, E) take no part in the order:
+ * the valid entries fill the front of sorted_*, offsets[E-1] counts them, and what lies behind them in sorted_* is
+ * left untouched (a caller that cannot rule such ids out pre-fills sorted_* with a sentinel). */
 size_t moe_sort_workspace_bytes(int64_t R, int E);
 int moe_sort_by_expert(const void* expert_idx, int in64, int64_t R, int E, int block_m, void* sorted_expert,
                        void* sorted_pos, int out64, void* counts, void* offsets, void* padded_blocks,
@@ -175,7 +182,8 @@ int moe_swiglu_bwd(const void* gate, const void* up, const void* dh, void* dgate
                    void* stream);
 
 /* ---- fused expert MLP: scattermoe_permute_and_compute, config_utils.py:99-185 ---------------------------------
- * bf16 only.  Weights in the reference's storage layout (sparse_mlp2.py:22-36 viewed as config_utils.py:31):
+ * bf16 or fp16 (`dtype`; the reference's `bf16` / `fp16` switches, megablocks_utils/shard_moe_utils.py:29-30,43-44), every
+ * tensor of a call in that one type.  Weights in the reference's storage layout (sparse_mlp2.py:22-36 viewed as config_utils.py:31):
  * w1, w3, w2 each (E, f, d) contiguous.  Adapters as the strided views of config_utils.py:48-56:
  * a1,a3 (E,d,r)  b1,b3 (E,r,f)  a2 (E,f,r)  b2 (E,r,d), strides {expert, second dim, third dim} in lora_strides[6][3]
  * (order a1,b1,a3,b3,a2,b2); all NULL = no adapters.
@@ -189,18 +197,18 @@ size_t moe_mlp_saved_bytes(int64_t R, int rank);
 int moe_mlp_fwd(const void* x, int64_t ldx, const void* w1, const void* w3, const void* w2, const void* const* lora,
                 const int64_t* lora_strides, int rank, float scaling, void* gate, void* up, void* h, void* y,
                 int64_t ldy, const void* pos, int pos64, const void* offsets, int off64, int E, int64_t R, int64_t d,
-                int64_t f, int fan_out, int y_grouped, void* saved, void* workspace, size_t workspace_bytes,
+                int64_t f, int fan_out, int y_grouped, int dtype, void* saved, void* workspace, size_t workspace_bytes,
                 void* stream);
 /* Backward of moe_mlp_fwd.  dy rows are addressed like y rows: row = dy_grouped ? m : pos[m] / dy_fan_out, and are
  * multiplied by row_scale[m] (fp32, may be NULL) -- this folds the combine's gate weights into the GEMM.
  * Outputs: dx_rows (R, d) written to row pos[m] (or m when dx_grouped), one row per assignment (the caller sums
- * the fan-out); adapter gradients in lora_grads (same order/strides convention as `lora`, dtype bf16). */
+ * the fan-out); adapter gradients in lora_grads (same order/strides convention as `lora`, same dtype). */
 int moe_mlp_bwd(const void* dy, int64_t lddy, int dy_grouped, int dy_fan_out, const float* row_scale, const void* x,
                 int64_t ldx, const void* w1, const void* w3, const void* w2, const void* const* lora,
                 const int64_t* lora_strides, void* const* lora_grads, const int64_t* lora_grad_strides, int rank,
                 float scaling, const void* gate, const void* up, const void* h, void* dgate, void* dup, void* dx_rows,
                 int64_t lddx, int dx_grouped, const void* pos, int pos64, const void* offsets, int off64, int E,
-                int64_t R, int64_t d, int64_t f, int fan_out, const void* saved, void* workspace,
+                int64_t R, int64_t d, int64_t f, int fan_out, int dtype, const void* saved, void* workspace,
                 size_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus

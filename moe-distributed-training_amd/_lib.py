@@ -9,6 +9,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmoe_hip.so")
 
+ABI_VERSION = 2   # MOE_HIP_ABI_VERSION of include/moe_hip.h this binding was written against
 MOE_BF16, MOE_F16, MOE_F32 = 0, 1, 2
 _DTYPES = {torch.bfloat16: MOE_BF16, torch.float16: MOE_F16, torch.float32: MOE_F32}
 
@@ -30,6 +31,7 @@ _SIGNATURES = {
     "moe_router_weight_grad_workspace_bytes": ("z", "lli"),
     "moe_router_weight_grad": ("i", "plppllliipzp"),
     "moe_gemm_debug_plan_blocks": ("l", "lili"),
+    "moe_gemm_debug_launch_count": ("l", ""),
     "moe_gemm_debug_plan": ("i", "piilllii" + "pp"),
     "moe_sort_workspace_bytes": ("z", "li"),
     "moe_sort_by_expert": ("i", "piliippippplpppzp"),
@@ -49,8 +51,8 @@ _SIGNATURES = {
     "moe_swiglu_bwd": ("i", "ppppplip"),
     "moe_mlp_workspace_bytes": ("z", "lilli"),
     "moe_mlp_saved_bytes": ("z", "li"),
-    "moe_mlp_fwd": ("i", "pl" + "ppp" + "pp" + "if" + "pppp" + "l" + "pi" + "pi" + "i" + "lll" + "ii" + "p" + "pzp"),
-    "moe_mlp_bwd": ("i", "plii" + "p" + "pl" + "ppp" + "pp" + "pp" + "if" + "ppp" + "pp" + "pli" + "pi" + "pi" + "i" + "lll" + "i" + "p" + "pzp"),
+    "moe_mlp_fwd": ("i", "pl" + "ppp" + "pp" + "if" + "pppp" + "l" + "pi" + "pi" + "i" + "lll" + "iii" + "p" + "pzp"),
+    "moe_mlp_bwd": ("i", "plii" + "p" + "pl" + "ppp" + "pp" + "pp" + "if" + "ppp" + "pp" + "pli" + "pi" + "pi" + "i" + "lll" + "ii" + "p" + "pzp"),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
@@ -62,12 +64,13 @@ def _load() -> ctypes.CDLL:
             f"{LIB_PATH} not found: the HIP extension must be built first "
             f"(python -c 'import __graft_entry__ as g; g.build()' or make -C {os.path.join(_HERE, 'csrc')})")
     lib = ctypes.CDLL(LIB_PATH)
+    lib.moe_hip_abi_version.restype = ctypes.c_int
+    if lib.moe_hip_abi_version() != ABI_VERSION:   # before the symbol table: an older library lacks entry points
+        raise ImportError(f"{LIB_PATH} has ABI version {lib.moe_hip_abi_version()}, this binding needs {ABI_VERSION}: rebuild the library")
     for name, (res, args) in _SIGNATURES.items():
         fn = getattr(lib, name)  # AttributeError if the library does not export a declared symbol
         fn.restype = ctypes.c_char_p if res == "s" else _CODES[res]
         fn.argtypes = [_CODES[c] for c in args]
-    if lib.moe_hip_abi_version() != 1:
-        raise ImportError("libmoe_hip.so ABI version mismatch")
     return lib
 
 

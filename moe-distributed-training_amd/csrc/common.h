@@ -43,6 +43,45 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi)
 }
 __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) { return (uint16_t)pack_bf16x2(f, 0.f); }
 
+// The matrix-core kernels are written once for both 16-bit storage types: a policy type says how 16 bits become a
+// float, how two floats are rounded (to nearest even) into a packed pair, and which 16x16x32 MFMA takes the
+// fragments.  Fragments travel as bf16x8_t whatever they hold (16 bytes per lane).
+typedef _Float16 moe_f16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 moe_f16x2_t __attribute__((ext_vector_type(2)));
+struct NumBf16 {
+    static constexpr int dtype = MOE_BF16;
+    static __device__ __forceinline__ float to_f32(uint16_t b) { return bf16_bits_to_f32(b); }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_bf16x2(lo, hi); }
+    static __device__ __forceinline__ uint16_t from_f32(float f) { return f32_to_bf16_bits(f); }
+    // rounds a pair to storage precision in place
+    static __device__ __forceinline__ void round2(float& a, float& b)
+    {
+        const uint32_t w = pack_bf16x2(a, b);
+        a = __uint_as_float(w << 16);
+        b = __uint_as_float(w & 0xffff0000u);
+    }
+    static __device__ __forceinline__ f32x4_t mfma(bf16x8_t a, bf16x8_t b, f32x4_t c) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0); }
+};
+struct NumF16 {
+    static constexpr int dtype = MOE_F16;
+    static __device__ __forceinline__ float to_f32(uint16_t b) { return (float)__builtin_bit_cast(_Float16, b); }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi)
+    {
+        const moe_f32x2_t v = {lo, hi};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, moe_f16x2_t));
+    }
+    static __device__ __forceinline__ uint16_t from_f32(float f) { return __builtin_bit_cast(uint16_t, (_Float16)f); }
+    static __device__ __forceinline__ void round2(float& a, float& b)
+    {
+        a = (float)(_Float16)a;
+        b = (float)(_Float16)b;
+    }
+    static __device__ __forceinline__ f32x4_t mfma(bf16x8_t a, bf16x8_t b, f32x4_t c)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(moe_f16x8_t, a), __builtin_bit_cast(moe_f16x8_t, b), c, 0, 0, 0);
+    }
+};
+
 template <typename T> struct Elem;
 template <> struct Elem<float> {
     static __device__ __forceinline__ float ld(const float* p) { return *p; }
@@ -129,6 +168,27 @@ __device__ __forceinline__ bool find_row_tile(const void* offsets, int off64, in
         else if ((dtype) == MOE_F32) { typedef float T; __VA_ARGS__; }                   \
         else return MOE_ERR_BAD_ARG;                                                     \
     } while (0)
+
+// Per-device caches (dynamic LDS opt-in done, compute-unit count) are indexed by the HIP device ordinal.
+constexpr int MOE_MAX_DEVICES = 64;
+static inline int moe_current_device()
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MOE_MAX_DEVICES) dev = 0;
+    return dev;
+}
+// compute units of the current device, looked up once per device
+static inline int moe_device_cus()
+{
+    static std::atomic<int> cus[MOE_MAX_DEVICES];
+    const int dev = moe_current_device();
+    int n = cus[dev];
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1) n = 256;
+        cus[dev] = n;
+    }
+    return n;
+}
 
 static inline int moe_launch_status()
 {

@@ -19,21 +19,13 @@
 #include "kernels.h"
 #include <type_traits>
 
-#ifndef SK_ORDER
-#define SK_ORDER __ATOMIC_ACQ_REL
-#endif
 #define EPI_IS_PAIR(e) ((e) == MOE_EPI_SWIGLU || (e) == MOE_EPI_SWIGLU_FUSED)
 constexpr int NXCD_HOST = 8;
+// compute units of the current device that the tile plan fills: a multiple of 8 (whole rounds are dealt out to the 8 XCDs)
 static int moe_num_cus()
 {
-    static std::atomic<int> cus{0};
-    if (cus == 0) {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1) n = 256;
-        n = n / NXCD_HOST * NXCD_HOST;     // the tile plan deals whole rounds out to the 8 XCDs
-        cus = n < NXCD_HOST ? NXCD_HOST : n;
-    }
-    return cus;
+    const int n = moe_device_cus() / NXCD_HOST * NXCD_HOST;
+    return n < NXCD_HOST ? NXCD_HOST : n;
 }
 
 namespace {
@@ -73,13 +65,13 @@ constexpr int INTERLEAVE_MIN_ROUNDS = 8;    // launches with at least this many 
 // awaited with explicit s_waitcnt vmcnt(n) below.
 typedef int i32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ i32x4_t make_buffer(const void* base)
+__device__ __forceinline__ i32x4_t make_buffer(const void* base, uint32_t num_records = 0xFFFFFFFFu)
 {
     const uint64_t a = (uint64_t)base;
     i32x4_t r;
     r.x = __builtin_amdgcn_readfirstlane((int)(uint32_t)a);
     r.y = __builtin_amdgcn_readfirstlane((int)(uint32_t)(a >> 32));   // stride field (bits 16..29 of this word) = 0: raw buffer
-    r.z = -1;                                                         // num_records: offsets are checked on the host
+    r.z = (int)num_records;                                           // a per-lane offset at or above this is out of range (loads return zeros); real offsets are checked on the host
     r.w = 0x00020000;                                                 // 32-bit data format
     return r;
 }
@@ -102,6 +94,7 @@ struct WorkItem {
     int split_item;            // exchange slot of this part (the slots of a tile are consecutive, in part order)
     int split_tile;            // counter of the split tile
     int mtile;                 // number of the row tile among all row tiles (experts in order, BM rows each)
+    int mt_in_group;           // number of the row tile within its expert's group (0: the group's first tile)
 };
 
 __device__ __forceinline__ WorkItem decode_work_item(const void* offsets, int off64, int E, int ntiles_n, int ktiles,
@@ -173,6 +166,7 @@ __device__ __forceinline__ WorkItem decode_work_item(const void* offsets, int of
         w.row0 = uniform_i64(row0);
         w.row1 = uniform_i64(row1);
         w.mtile = __builtin_amdgcn_readfirstlane((int)(before + mt));
+        w.mt_in_group = __builtin_amdgcn_readfirstlane((int)mt);
         w.valid = true;
     } else {
         int64_t start = 0, id = t, mtiles_before = 0;
@@ -185,6 +179,7 @@ __device__ __forceinline__ WorkItem decode_work_item(const void* offsets, int of
                 w.nt = (int)(id / mte);
                 const int64_t mt = id % mte;
                 w.mtile = (int)(mtiles_before + mt);
+                w.mt_in_group = (int)mt;
                 w.row0 = start + mt * BM;
                 w.row1 = (w.row0 + BM < end) ? w.row0 + BM : end;
                 w.valid = true;
@@ -214,7 +209,9 @@ __global__ void gemm_plan_kernel(const void* offsets, int off64, int E, int ntil
     }
 }
 
-template <bool NN, int EPI>
+// KTAIL: K is not a multiple of the 64-wide K tile (but of 8): the last tile of every K segment is partial, and the loads
+// that would reach past K fetch zeros instead.  A variant of its own so that the loop for whole tiles carries none of it.
+template <bool NN, int EPI, typename Num, bool KTAIL>
 __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGemmParams p)
 {
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
@@ -227,7 +224,7 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
 
     // ---- work item -> (expert, n tile, m tile, K part)
     const int ntiles_n = (EPI_IS_PAIR(EPI)) ? (int)((p.N + BN / 2 - 1) / (BN / 2)) : (int)((p.N + BN - 1) / BN);
-    const int ktiles_seg = (int)(p.K / BK);
+    const int ktiles_seg = KTAIL ? (int)((p.K + BK - 1) / BK) : (int)(p.K / BK);
     const int ktiles = ktiles_seg * p.nseg;
     const WorkItem item = decode_work_item(p.offsets, p.off64, p.E, ntiles_n, ktiles, p.max_split, p.num_cus);
     if (!item.valid) return;
@@ -264,12 +261,15 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
         const int c = (lane & 7) ^ ((r >> 1) & 7);
         a_off[j] = (uint32_t)(((s_inrow[r] - a_row_base) * p.ldx + c * 8) * 2);
     }
-    const i32x4_t a_buf0 = make_buffer(p.X[0] + a_row_base * p.ldx), a_buf1 = make_buffer((p.X[1] ? p.X[1] : p.X[0]) + a_row_base * p.ldx);
+    // (KTAIL: the masked loads of a partial K tile use the offset OUT_OF_RANGE, which must lie at or above the descriptors'
+    // range -- with the full 32-bit range it would be a valid offset and the load would touch memory 4 GiB past the base)
+    constexpr uint32_t LOAD_RANGE = KTAIL ? 0x80000000u : 0xFFFFFFFFu;
+    const i32x4_t a_buf0 = make_buffer(p.X[0] + a_row_base * p.ldx, LOAD_RANGE), a_buf1 = make_buffer((p.X[1] ? p.X[1] : p.X[0]) + a_row_base * p.ldx, LOAD_RANGE);
     // B: offsets within this expert's matrix.  For the SwiGLU pair image rows [0,128) come from W[0] and [128,256)
     // from W[1], which are whole load instructions (the first and second half of a wave's LPT); otherwise W[0] / W[1]
     // are the two K segments.
     uint32_t b_off[LPT];
-    const i32x4_t b_buf0 = make_buffer(p.W[0] + (int64_t)expert * p.swe), b_buf1 = make_buffer((p.W[1] ? p.W[1] : p.W[0]) + (int64_t)expert * p.swe);
+    const i32x4_t b_buf0 = make_buffer(p.W[0] + (int64_t)expert * p.swe, LOAD_RANGE), b_buf1 = make_buffer((p.W[1] ? p.W[1] : p.W[0]) + (int64_t)expert * p.swe, LOAD_RANGE);
     if (!NN) {
         // B image as A: row = n (BN rows of 64 k)
 #pragma unroll
@@ -372,12 +372,27 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
     // stored or summed); the wait counts of the main loop only ever leave weight instructions in flight, which are never dropped,
     // so they do not depend on how many activation instructions were.
     const int live_rows = (nrows + 31) / 32 * 32;
+    // Partial last K tile (KTAIL): a load whose 8 k (K-contiguous images) or whose k row (N-contiguous image) lies at or past
+    // K gets a per-lane offset beyond the descriptor's range (LOAD_RANGE, 2 GiB in this variant) -- the hardware then writes
+    // zeros to LDS and touches no memory.
+    // The range check looks at the per-lane offset, so the K advance moves from the scalar offset into it for that tile.
+    // The 16-byte chunk a lane fetches of a K-contiguous row is (lane & 7) ^ ((row >> 1) & 7), the same in all of a wave's
+    // load instructions (their rows differ by multiples of 64).
+    constexpr uint32_t OUT_OF_RANGE = 0xFFFFFFF0u;
+    const uint32_t ktail_kq = (uint32_t)(((lane & 7) ^ (((lane >> 4) + 4 * (wave & 1)) & 7)) * 8);
     auto issue_a = [&](int kt, int jj, int stage, bool ragged) {
         kt = __builtin_amdgcn_readfirstlane(kt < ke ? kt : ke - 1);
         const int seg = (kt >= ktiles_seg) ? 1 : 0;
         const uint32_t k0 = (uint32_t)(kt - seg * ktiles_seg) * BK;
+        if constexpr (KTAIL) {
+            uint32_t voff = a_off[jj], soff = k0 * 2;
+            if (k0 + BK > (uint32_t)p.K) { voff = (k0 + ktail_kq < (uint32_t)p.K) ? voff + soff : OUT_OF_RANGE; soff = 0; }
+            if (!ragged || (jj * NWAVES + wave) * 8 < live_rows)
+                load_to_lds_16(seg ? a_buf1 : a_buf0, voff, soff, smem_u + stage * A_STAGE_BYTES + jj * (NWAVES * 1024));
+        } else {
         if (!ragged || (jj * NWAVES + wave) * 8 < live_rows)
             load_to_lds_16(seg ? a_buf1 : a_buf0, a_off[jj], k0 * 2, smem_u + stage * A_STAGE_BYTES + jj * (NWAVES * 1024));
+        }
     };
     // the same instruction slot for the slab image (the activation image of tile ke)
     auto issue_slab = [&](int jj, int stage) {
@@ -390,7 +405,18 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
         const int seg = (kt >= ktiles_seg) ? 1 : 0;
         const uint32_t k0 = (uint32_t)(kt - seg * ktiles_seg) * BK;
         const bool second = (EPI_IS_PAIR(EPI)) ? (idx >= LPT / 2) : (seg != 0);
+        if constexpr (KTAIL) {
+            uint32_t voff = b_off[idx], soff = NN ? k0 * (uint32_t)p.ldw * 2 : k0 * 2;
+            if (k0 + BK > (uint32_t)p.K) {
+                // K-contiguous image: this lane's 8 k as for the activation image; N-contiguous image: the lane's whole k row
+                const bool in = NN ? k0 + (uint32_t)((idx * NWAVES + wave) * 2 + (lane >> 5)) < (uint32_t)p.K : k0 + ktail_kq < (uint32_t)p.K;
+                voff = in ? voff + soff : OUT_OF_RANGE;
+                soff = 0;
+            }
+            load_to_lds_16(second ? b_buf1 : b_buf0, voff, soff, smem_u + B_REGION + stage * B_STAGE_BYTES + idx * (NWAVES * 1024));
+        } else {
         load_to_lds_16(second ? b_buf1 : b_buf0, b_off[idx], NN ? k0 * (uint32_t)p.ldw * 2 : k0 * 2, smem_u + B_REGION + stage * B_STAGE_BYTES + idx * (NWAVES * 1024));
+        }
     };
 
     // fragment readers (LDS -> registers), one 16-wide block each.  Accumulator tiles are kept transposed -- the weight fragment is the
@@ -463,14 +489,17 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
         // A tail tile of at most two row blocks has next to no MFMA work and would run through K several times faster than
         // the full row tiles that share its weight tiles: the weight tiles it fetches are then gone from L2 again before
         // those arrive (measured on the gate/up launch: 0.8 GB more fetched from memory with three such tails), and its
-        // requests compete with theirs.  Its waves therefore take at least PACE_CYCLES per K tile (a full tile cannot
-        // take less: 2048 cycles are its MFMAs alone), which keeps it just ahead of them -- close enough to act as their
+        // requests compete with theirs.  The waves of such a tile therefore take at least PACE_CYCLES per K tile (a full tile
+        // cannot take less: 2048 cycles are its MFMAs alone), which keeps it just ahead of them -- close enough to act as their
         // prefetcher.  Measured over eight routing draws of 8192 rows: the launches of few rounds 1-2 % faster; the gate/up
         // launch, whose sixteen rounds are bound by the sum of the tiles' times, 2 % slower than with unpaced tails --
-        // the price of not fetching those weight tiles twice.
+        // the price of not fetching those weight tiles twice.  The copy of the loop is chosen per wave (its live blocks);
+        // whether it paces is decided per tile: only a tail that follows full row tiles of its group shares weight tiles
+        // with anybody -- a group's first tile (small batches, many experts with a few rows each) runs unpaced.
         constexpr bool PACED = !FULL && NBLK <= 2;
+        const bool pace = PACED && item.mt_in_group > 0;
         constexpr int64_t PACE_CYCLES = 2048;
-        int64_t pace_t0 = PACED ? (int64_t)__builtin_readcyclecounter() : 0;
+        int64_t pace_t0 = pace ? (int64_t)__builtin_readcyclecounter() : 0;
         // one K tile; SLAB: the activation loads it requests (for tile kt+2) fetch the slab image instead
         auto tile = [&](int kt, auto slab_tag) {
             constexpr bool SLAB = decltype(slab_tag)::value;
@@ -486,7 +515,7 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
                 // ra / rb: where the fragments of the next half step come from; for the last one of a tile, the first of
                 // the next tile.  (After the last tile this fetches fragments nobody uses.)
                 if (hs == 3) {
-                    if (PACED) {   // (see PACE_CYCLES; a sleep is 128 cycles, so the count bounds the wait whatever the counter's rate)
+                    if (pace) {   // (see PACE_CYCLES; a sleep is 128 cycles, so the count bounds the wait whatever the counter's rate)
                         for (int n = 0; n < 24 && (int64_t)__builtin_readcyclecounter() - pace_t0 < PACE_CYCLES; ++n) __builtin_amdgcn_s_sleep(2);
                         pace_t0 = (int64_t)__builtin_readcyclecounter();
                     }
@@ -533,7 +562,7 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
                         __builtin_amdgcn_sched_barrier(0);
                     }
                     if (mh * MBH + mb < NBLK)
-                        acc[mh * MBH + mb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bf[cur_b][nb], af[cur_a][mb], acc[mh * MBH + mb][nb], 0, 0, 0);
+                        acc[mh * MBH + mb][nb] = Num::mfma(bf[cur_b][nb], af[cur_a][mb], acc[mh * MBH + mb][nb]);
                 }
                 __builtin_amdgcn_s_setprio(0);
                 __builtin_amdgcn_sched_barrier(0);
@@ -586,7 +615,9 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
             }
         __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave's stores are acknowledged
         __syncthreads();                      // ... and every wave's: the partial is visible
-        if (tid == 0) *s_arrival = __hip_atomic_fetch_add(&p.sk_counters[ti], 1, SK_ORDER, __HIP_MEMORY_SCOPE_AGENT);
+        // release + acquire at agent scope: the parts of a tile run on different XCDs with separate L2 caches, and the part that
+        // counts last must find every earlier part's partial (a relaxed increment lets it read stale lines)
+        if (tid == 0) *s_arrival = __hip_atomic_fetch_add(&p.sk_counters[ti], 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
         if (*s_arrival != nparts - 1) return;
         if (tid == 0) __hip_atomic_store(&p.sk_counters[ti], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // clean for the next launch
@@ -687,7 +718,7 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
 #pragma unroll
                         for (int nb = 0; nb < NB; ++nb)
                             if (group_of[s] < 0 || nb / NBH == group_of[s])
-                                acc[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(sb[s][nb], sa[s][mb], acc[mb][nb], 0, 0, 0);
+                                acc[mb][nb] = Num::mfma(sb[s][nb], sa[s][mb], acc[mb][nb]);
                     }
             }
         }
@@ -706,8 +737,8 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
     }
     auto pack4 = [](float a, float b, float c, float d) {
         uint2 v;
-        v.x = pack_bf16x2(a, b);
-        v.y = pack_bf16x2(c, d);
+        v.x = Num::pack2(a, b);
+        v.y = Num::pack2(c, d);
         return v;
     };
     // Staging image of SW columns per row (SW*2 bytes, SW/8 chunks of 16 bytes).  256 bytes span the 64 LDS banks, so
@@ -771,9 +802,10 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
             for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
                 for (int r = 0; r < 4; r += 2) {
-                    const uint32_t w2 = pack_bf16x2(acc[mb][nb][r], acc[mb][nb][r + 1]);
-                    acc[mb][nb][r] = __uint_as_float(w2 << 16);
-                    acc[mb][nb][r + 1] = __uint_as_float(w2 & 0xffff0000u);
+                    float a_ = acc[mb][nb][r], b_ = acc[mb][nb][r + 1];
+                    Num::round2(a_, b_);
+                    acc[mb][nb][r] = a_;
+                    acc[mb][nb][r + 1] = b_;
                 }
 #pragma unroll
         for (int pass = 0; pass < 3; ++pass) {
@@ -805,7 +837,7 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
                 for (int mb = 0; mb < MB; ++mb) {
                     const bf16x8_t hf = *(const bf16x8_t*)(stg + (mb * 16 + (lane & 15)) * (WTN / 2 * 2) + (((lane >> 4) ^ ((lane >> 2) & 3)) << 4));
                     const f32x4_t z = {0.f, 0.f, 0.f, 0.f};
-                    const f32x4_t d_ = __builtin_amdgcn_mfma_f32_16x16x32_bf16(hf, cb, z, 0, 0, 0);
+                    const f32x4_t d_ = Num::mfma(hf, cb, z);
                     *(f32x4_t*)(park + (mb * 64 + lane) * 4) = d_;
                 }
             }
@@ -954,17 +986,17 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
                     float og[2], ou[2], hh[2];
 #pragma unroll
                     for (int t = 0; t < 2; ++t) {
-                        const float g = bf16_bits_to_f32((uint16_t)(gg[w2] >> (t * 16)));
-                        const float u = bf16_bits_to_f32((uint16_t)(uu[w2] >> (t * 16)));
-                        const float dh = bf16_bits_to_f32((uint16_t)(dh8[w2] >> (t * 16)));
+                        const float g = Num::to_f32((uint16_t)(gg[w2] >> (t * 16)));
+                        const float u = Num::to_f32((uint16_t)(uu[w2] >> (t * 16)));
+                        const float dh = Num::to_f32((uint16_t)(dh8[w2] >> (t * 16)));
                         const float sg = sigmoid_f(g);
                         og[t] = dh * u * sg * (1.f + g * (1.f - sg));
                         ou[t] = dh * g * sg;
                         hh[t] = g * sg * u;
                     }
-                    og8[q][w2] = pack_bf16x2(og[0], og[1]);
-                    ou8[q][w2] = pack_bf16x2(ou[0], ou[1]);
-                    if (FUSED) hh8[q][w2] = pack_bf16x2(hh[0], hh[1]);
+                    og8[q][w2] = Num::pack2(og[0], og[1]);
+                    ou8[q][w2] = Num::pack2(ou[0], ou[1]);
+                    if (FUSED) hh8[q][w2] = Num::pack2(hh[0], hh[1]);
                     // Rows past the group must enter the contractions as exact zeros.  Their gate / up read as zeros, but
                     // their dh need not be finite: the accumulators of row blocks without real rows can hold anything (an
                     // MFMA that the compiler left under an execution mask instead of a branch runs all the same -- the
@@ -1018,13 +1050,13 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
                     const int gen = mat & 1;
 #pragma unroll
                     for (int ib = 0; ib < IBLK; ++ib)
-                        rcd[mat][ib] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[gen][ib], pf[gen], rcd[mat][ib], 0, 0, 0);
+                        rcd[mat][ib] = Num::mfma(vf[gen][ib], pf[gen], rcd[mat][ib]);
                     if (mat < CC_MATS) {
 #pragma unroll
                         for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
                             for (int ks = 0; ks < CC_KS; ++ks)
-                                ccd[mat][rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cf[gen][rb][ks], cbf[mat][ks], ccd[mat][rb], 0, 0, 0);
+                                ccd[mat][rb] = Num::mfma(cf[gen][rb][ks], cbf[mat][ks], ccd[mat][rb]);
                     }
                 };
                 queue(0);
@@ -1111,14 +1143,15 @@ int64_t plan_grid(int64_t R, int E, int ntiles_n, int ncu)
     return (grid + NXCD - 1) / NXCD * NXCD;
 }
 
-template <bool NN, int EPI> int launch_variant(const MoeGemmParams& p, int64_t R, hipStream_t stream)
+template <bool NN, int EPI, typename Num, bool KTAIL> int launch_typed(const MoeGemmParams& p, int64_t R, hipStream_t stream)
 {
-    static std::atomic<bool> attr_set{false};   // forward and backward may call from different host threads
-    auto kern = grouped_gemm_mfma_kernel<NN, EPI>;
-    if (!attr_set) {
+    static std::atomic<bool> attr_set[MOE_MAX_DEVICES];   // per device; forward and backward may call from different host threads
+    auto kern = grouped_gemm_mfma_kernel<NN, EPI, Num, KTAIL>;
+    const int dev = moe_current_device();
+    if (!attr_set[dev]) {
         if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess)
             return MOE_ERR_LAUNCH;
-        attr_set = true;
+        attr_set[dev] = true;
     }
     const int ntiles_n = (EPI_IS_PAIR(EPI)) ? (int)((p.N + BN / 2 - 1) / (BN / 2)) : (int)((p.N + BN - 1) / BN);
     MoeGemmParams q = p;
@@ -1134,6 +1167,18 @@ template <bool NN, int EPI> int launch_variant(const MoeGemmParams& p, int64_t R
     return moe_launch_status();
 }
 
+// the kernel variant for the launch's 16-bit storage type
+template <bool NN, int EPI> int launch_variant(const MoeGemmParams& p, int64_t R, hipStream_t stream)
+{
+    if (p.K % BK != 0) {   // a partial last K tile: the plain epilogue only (the fused layer's shapes are whole tiles)
+        if constexpr (EPI == MOE_EPI_STORE)
+            return p.f16 ? launch_typed<NN, EPI, NumF16, true>(p, R, stream) : launch_typed<NN, EPI, NumBf16, true>(p, R, stream);
+        else
+            return MOE_ERR_UNSUPPORTED;
+    }
+    return p.f16 ? launch_typed<NN, EPI, NumF16, false>(p, R, stream) : launch_typed<NN, EPI, NumBf16, false>(p, R, stream);
+}
+
 }  // namespace
 
 
@@ -1147,11 +1192,11 @@ int64_t moe_gemm_plan_blocks(int64_t R, int E, int64_t N, int pair) { return pla
 int moe_launch_gemm_plan(const void* offsets, int off64, int E, int64_t R, int64_t K, int64_t N, int pair, int nseg, int* out,
                          hipStream_t stream)
 {
-    if (K % BK != 0 || nseg < 1 || nseg > 2) return MOE_ERR_UNSUPPORTED;
+    if (K < BK || nseg < 1 || nseg > 2) return MOE_ERR_UNSUPPORTED;
     const int ntiles_n = plan_ntiles_n(N, pair);
     const int64_t grid = plan_grid(R, E, ntiles_n, moe_num_cus());
     hipLaunchKernelGGL(gemm_plan_kernel, dim3((unsigned)grid), dim3(64), 0, stream, offsets, off64, E, ntiles_n,
-                       (int)(K / BK) * nseg, moe_gemm_max_split(pair != 0), moe_num_cus(), out);
+                       (int)((K + BK - 1) / BK) * nseg, moe_gemm_max_split(pair != 0), moe_num_cus(), out);
     return moe_launch_status();
 }
 
@@ -1173,7 +1218,8 @@ void moe_gemm_sk_attach(MoeGemmParams& p, void* ws, int64_t, int, int64_t)
 bool moe_gemm_mfma_supported(const MoeGemmParams& p, int64_t R)
 {
     auto al16 = [](const void* q) { return q == nullptr || ((uintptr_t)q % 16) == 0; };
-    if (p.K <= 0 || p.K % BK != 0 || p.N % 8 != 0 || p.ldx % 8 != 0 || p.ldw % 8 != 0 || p.swe % 8 != 0) return false;
+    // whole 64-wide K tiles run through the main loop (at least one), a remainder (multiple of 8) through the tail step
+    if (p.K < BK || p.K % 8 != 0 || p.N % 8 != 0 || p.ldx % 8 != 0 || p.ldw % 8 != 0 || p.swe % 8 != 0) return false;
     if (!al16(p.X[0]) || !al16(p.X[1]) || !al16(p.W[0]) || !al16(p.W[1])) return false;
     for (int i = 0; i < MOE_MAX_SLABS; ++i)
         if (!al16(p.Q[i]) || !al16(p.LB[i])) return false;
@@ -1184,18 +1230,23 @@ bool moe_gemm_mfma_supported(const MoeGemmParams& p, int64_t R)
     (void)R;
     const int fo = p.fan_out > 0 ? p.fan_out : 1;
     const int64_t x_rows = p.x_grouped ? BM : (R + fo - 1) / fo;
-    const int64_t limit = (int64_t)1 << 32;
+    // (a partial last K tile masks its loads through the descriptor's range, which that kernel variant sets to 2 GiB)
+    const int64_t limit = (p.K % BK != 0) ? (int64_t)1 << 31 : (int64_t)1 << 32;
     if ((x_rows * p.ldx + p.K) * 2 >= limit) return false;
     if (((p.nn ? p.K : p.N) * p.ldw + (p.nn ? p.N : p.K)) * 2 >= limit) return false;
-    if ((BM * p.ldy + p.N) * 2 >= limit / 2) return false;
-    if ((p.epi == MOE_EPI_SWIGLU_BWD || p.epi == MOE_EPI_SWIGLU_BWD_FUSED) && (BM * p.ldh + p.N) * 2 >= limit / 2) return false;
+    if ((BM * p.ldy + p.N) * 2 >= ((int64_t)1 << 31)) return false;
+    if ((p.epi == MOE_EPI_SWIGLU_BWD || p.epi == MOE_EPI_SWIGLU_BWD_FUSED) && (BM * p.ldh + p.N) * 2 >= ((int64_t)1 << 31)) return false;
     return true;
 }
+
+static std::atomic<int64_t> g_mfma_launches{0};
+int64_t moe_gemm_mfma_launch_count() { return g_mfma_launches; }
 
 int moe_launch_gemm_mfma(const MoeGemmParams& p, int64_t R, hipStream_t stream)
 {
     if (R == 0 || p.N == 0) return MOE_OK;
     if (!moe_gemm_mfma_supported(p, R)) return MOE_ERR_UNSUPPORTED;
+    ++g_mfma_launches;
     if (p.epi == MOE_EPI_STORE) return p.nn ? launch_variant<true, MOE_EPI_STORE>(p, R, stream) : launch_variant<false, MOE_EPI_STORE>(p, R, stream);
     if (p.epi == MOE_EPI_SWIGLU) return p.nn ? MOE_ERR_UNSUPPORTED : launch_variant<false, MOE_EPI_SWIGLU>(p, R, stream);
     if (p.epi == MOE_EPI_SWIGLU_FUSED) {

@@ -40,6 +40,7 @@ __device__ __forceinline__ void load_to_lds_16(i32x4_t rsrc, uint32_t lane_off, 
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_addr), "v"(lane_off), "s"(rsrc) : "memory", "m0");
 }
 
+template <typename Num>
 __global__ void __launch_bounds__(NTHREADS) grouped_xty_mfma_kernel(const MoeXtyParams p)
 {
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
@@ -190,7 +191,7 @@ __global__ void __launch_bounds__(NTHREADS) grouped_xty_mfma_kernel(const MoeXty
                         issue_one(load_kt, g / LOAD_GAP);
                         __builtin_amdgcn_sched_barrier(0);
                     }
-                    acc[mh * MBH + mb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bf[cur_b][nb], af[cur_a][mb], acc[mh * MBH + mb][nb], 0, 0, 0);
+                    acc[mh * MBH + mb][nb] = Num::mfma(bf[cur_b][nb], af[cur_a][mb], acc[mh * MBH + mb][nb]);
                 }
                 __builtin_amdgcn_s_setprio(0);
                 __builtin_amdgcn_sched_barrier(0);
@@ -213,8 +214,8 @@ __global__ void __launch_bounds__(NTHREADS) grouped_xty_mfma_kernel(const MoeXty
         for (int nb = 0; nb < NB; ++nb) {
             const int m = mb * 16 + mrow, ncol = nb * 16 + nq;
             uint2 v;
-            v.x = pack_bf16x2(acc[mb][nb][0], acc[mb][nb][1]);
-            v.y = pack_bf16x2(acc[mb][nb][2], acc[mb][nb][3]);
+            v.x = Num::pack2(acc[mb][nb][0], acc[mb][nb][1]);
+            v.y = Num::pack2(acc[mb][nb][2], acc[mb][nb][3]);
             *(uint2*)(stg + m * (WTN * 2) + ((((ncol >> 3) ^ (m >> 1)) & (CPR - 1)) << 4) + ((ncol >> 2) & 1) * 8) = v;
         }
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's staging writes have landed
@@ -252,15 +253,17 @@ int moe_launch_xty_mfma(const MoeXtyParams& p, int64_t R, hipStream_t stream)
 {
     if (p.E < 1) return MOE_ERR_BAD_ARG;
     if (!moe_xty_mfma_supported(p, R)) return MOE_ERR_UNSUPPORTED;
-    static std::atomic<bool> attr_set{false};   // forward and backward may call from different host threads
-    if (!attr_set) {
-        if (hipFuncSetAttribute((const void*)grouped_xty_mfma_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess)
+    static std::atomic<bool> attr_set[MOE_MAX_DEVICES];   // per device; forward and backward may call from different host threads
+    const int dev = moe_current_device();
+    if (!attr_set[dev]) {
+        if (hipFuncSetAttribute((const void*)grouped_xty_mfma_kernel<NumBf16>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess ||
+            hipFuncSetAttribute((const void*)grouped_xty_mfma_kernel<NumF16>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess)
             return MOE_ERR_LAUNCH;
-        attr_set = true;
+        attr_set[dev] = true;
     }
     const int64_t per_e = ((p.K + BM - 1) / BM) * ((p.N + BN - 1) / BN);
     const int64_t grid = (per_e + NXCD - 1) / NXCD * p.E * NXCD;   // an eighth of every expert's tiles per XCD
     if (grid > 0x7fffffff) return MOE_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL(grouped_xty_mfma_kernel, dim3((unsigned)grid), dim3(NTHREADS), LDS_BYTES, stream, p);
+    hipLaunchKernelGGL(p.f16 ? grouped_xty_mfma_kernel<NumF16> : grouped_xty_mfma_kernel<NumBf16>, dim3((unsigned)grid), dim3(NTHREADS), LDS_BYTES, stream, p);
     return moe_launch_status();
 }

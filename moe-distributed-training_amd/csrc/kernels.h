@@ -54,6 +54,7 @@ struct MoeGemmParams {
     int x_grouped;
     int y_grouped;
     int epi;
+    int f16;                // operands and outputs are IEEE half instead of bfloat16
     int y_wide;             // scattered output rows need 64-bit addresses (Y spans 2 GiB or more), set by the launcher
     int max_split;          // K parts a tile of the last round may be cut into (1, 2 or 4), set by the launcher
     int num_cus;            // compute units the tile plan fills (a multiple of 8), set by the launcher
@@ -74,6 +75,7 @@ size_t moe_gemm_sk_bytes(int64_t R, int E, int64_t N);
 void moe_gemm_sk_attach(MoeGemmParams& p, void* ws, int64_t R, int E, int64_t N);
 bool moe_gemm_mfma_supported(const MoeGemmParams& p, int64_t R);
 int moe_launch_gemm_mfma(const MoeGemmParams& p, int64_t R, hipStream_t stream);
+int64_t moe_gemm_mfma_launch_count();   // test aid: matrix-core grouped GEMM launches enqueued by this process so far
 
 // weight gradient DW[e] = X_e^T DY_e on the matrix cores (bf16; unit column strides)
 struct MoeXtyParams {
@@ -87,6 +89,7 @@ struct MoeXtyParams {
     int off64;
     int E;
     int64_t K, N;
+    int f16;                // operands and output are IEEE half instead of bfloat16
 };
 bool moe_xty_mfma_supported(const MoeXtyParams& p, int64_t R);
 int moe_launch_xty_mfma(const MoeXtyParams& p, int64_t R, hipStream_t stream);
@@ -100,7 +103,7 @@ int moe_launch_generic_xty(const void* X, int64_t sxm, int64_t sxk, const void* 
                            int64_t soe, int64_t sok, int64_t son, const void* offsets, int off64, int E, int64_t K,
                            int64_t N, float scale, int dtype, hipStream_t stream);
 
-// low-rank helpers (bf16, rank <= 16)
+// low-rank helpers (16-bit storage: bf16, or IEEE half when f16 != 0; rank <= 16)
 // a batch of pack jobs sharing E: src strides {expert, k, r}, dst as moe_launch_pack_lora
 constexpr int MOE_PACK_MAX_JOBS = 12;
 struct MoePackJob { const uint16_t* src; int64_t se, sk, sr; uint16_t* dst; int64_t K; int transpose; int rank; };   // rank <= 16 columns, zero padded to 16
@@ -110,33 +113,33 @@ int moe_launch_pack_lora(const void* src, int64_t se, int64_t sk, int64_t sr, vo
                          int transpose, hipStream_t stream);
 int moe_launch_rows_lora(const void* X, int64_t ldx, const void* At, void* Q, void* Qt, int64_t ldqt, const void* pos,
                          int pos64, const void* offsets, int off64, int E, int64_t R, int64_t K, int fan_out,
-                         int x_grouped, float scaling, const float* qt_row_scale, hipStream_t stream);
+                         int x_grouped, float scaling, const float* qt_row_scale, hipStream_t stream, int f16 = 0);
 // two products over the same rows in one launch (X2 == nullptr: only the first)
 // q_scaled (optional): a third output of the first product, [R][16] like Q but multiplied by qt_row_scale like Qt
 int moe_launch_rows_lora2(const void* X, const void* X2, int64_t ldx, const void* At, const void* At2, void* Q, void* Q2,
                           void* Qt, void* Qt2, int64_t ldqt, const void* pos, int pos64, const void* offsets, int off64,
                           int E, int64_t R, int64_t K, int fan_out, int x_grouped, float scaling,
-                          const float* qt_row_scale, hipStream_t stream, void* q_scaled = nullptr);
+                          const float* qt_row_scale, hipStream_t stream, void* q_scaled = nullptr, int f16 = 0);
 size_t moe_xtp_workspace_bytes(int64_t R, int E, int64_t K);
 // Q[m][r] = bf16(scaling * sum over ntiles column-tile partials [ntiles][R][16]) and its transposed copy Qt[r][m], for one or
 // two products (partial2 == nullptr: one)
 int moe_launch_cc_reduce2(const float* partial, const float* partial2, int ntiles, int64_t R, float scaling, void* Q, void* Q2,
-                          void* Qt, void* Qt2, int64_t ldqt, hipStream_t stream);
+                          void* Qt, void* Qt2, int64_t ldqt, hipStream_t stream, int f16 = 0);
 // the reduction half of moe_launch_xtp2 alone, for partials [row tile of 256][K][16] that another kernel produced
 // (partial2 == nullptr: only the first)
 int moe_launch_xtp_reduce2(const float* partial, const float* partial2, void* out, void* out2, const int64_t* so,
                            const int64_t* so2, int rank, int rank2, const void* offsets, int off64, int E, int64_t K,
-                           float scale, hipStream_t stream);
+                           float scale, hipStream_t stream, int f16 = 0);
 // two reductions over the same rows in one launch pair (X2 == nullptr: only the first); so / so2: output strides
 // {expert, k, r}; rank / rank2: columns each writes; needs twice moe_xtp_workspace_bytes when X2 is given
 int moe_launch_xtp2(const void* X, const void* X2, int64_t ldx, const void* pos, int pos64, int fan_out, const void* Pt,
                     const void* Pt2, int64_t ldpt, const float* p_row_scale, void* out, void* out2, const int64_t* so,
                     const int64_t* so2, int rank, int rank2, const void* offsets, int off64, int E, int64_t R, int64_t K,
-                    float scale, void* workspace, size_t workspace_bytes, hipStream_t stream);
+                    float scale, void* workspace, size_t workspace_bytes, hipStream_t stream, int f16 = 0);
 int moe_launch_xtp(const void* X, int64_t ldx, const void* pos, int pos64, int fan_out, const void* Pt, int64_t ldpt,
                    const float* p_row_scale, void* out, int64_t soe, int64_t sok, int64_t sor, int rank,
                    const void* offsets, int off64, int E, int64_t R, int64_t K, float scale, void* workspace,
-                   size_t workspace_bytes, hipStream_t stream);
+                   size_t workspace_bytes, hipStream_t stream, int f16 = 0);
 
 // router + integer pipeline
 int moe_launch_router_logits(const void* x, int64_t ldx, const void* wg, int64_t ldw, int dtype, float* logits,

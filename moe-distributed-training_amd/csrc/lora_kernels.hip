@@ -10,12 +10,14 @@
 
 namespace {
 
+// (fragment order covers K rounded up to whole 32-wide fragments; positions at or past K hold zeros, so a consumer may
+// feed them anything finite)
 __global__ void pack_lora_kernel(const uint16_t* __restrict__ src, int64_t se, int64_t sk, int64_t sr,
-                                 uint16_t* __restrict__ dst, int64_t K, int rank, int transpose, int64_t total)
+                                 uint16_t* __restrict__ dst, int64_t K, int64_t Kimg, int rank, int transpose, int64_t total)
 {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= total) return;
-    const int64_t e = i / (K * 16), rem = i % (K * 16);
+    const int64_t e = i / (Kimg * 16), rem = i % (Kimg * 16);
     int64_t k;
     int r;
     if (transpose) {   // fragment order: one 16x16x32 operand fragment is 1 KiB of consecutive memory
@@ -24,7 +26,7 @@ __global__ void pack_lora_kernel(const uint16_t* __restrict__ src, int64_t se, i
         r = lane & 15;
         k = kb * 32 + 8 * (lane >> 4) + t;
     } else { k = rem / 16; r = (int)(rem % 16); }           // dst[e][k][r]
-    dst[i] = (r < rank) ? src[e * se + k * sk + r * sr] : (uint16_t)0;
+    dst[i] = (r < rank && k < K) ? src[e * se + k * sk + r * sr] : (uint16_t)0;
 }
 
 // several pack jobs in one launch (blockIdx.y selects the job): the six factors of an MLP block are a few MB in total,
@@ -92,7 +94,7 @@ static_assert(RL_KSTEPS == RL_WAVES, "one K step per wave and stage");
 struct RowsLoraJob { const uint16_t* X; const uint16_t* Af; uint16_t* Q; uint16_t* Qt; uint16_t* Qs; };   // Qs: optional row-major copy scaled like Qt
 // ROWS = 32 rows per workgroup, or 16 when a launch of 32-row tiles would leave most compute units with a single
 // workgroup (and so with too few loads in flight)
-template <int ROWS>
+template <int ROWS, typename Num>
 __global__ void __launch_bounds__(RL_THREADS) rows_lora_kernel(const RowsLoraJob job0, const RowsLoraJob job1, int64_t ldx,
                                                                int64_t ldqt, const void* __restrict__ pos, int pos64,
                                                                const void* __restrict__ offsets, int off64, int E,
@@ -125,9 +127,9 @@ __global__ void __launch_bounds__(RL_THREADS) rows_lora_kernel(const RowsLoraJob
         rowptr[q] = X + in_row * ldx;
     }
     const uint32_t lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)LDS_PTR(smem));
-    const uint16_t* abase = Af + (int64_t)expert * K * 16;
+    const int64_t nksteps = (K + 31) / 32;   // the adapter image is zero beyond K: a partial last step takes whatever x the lanes past the row's end re-read
+    const uint16_t* abase = Af + (int64_t)expert * nksteps * 512;
     const int nstages = (int)((K + RL_KC - 1) / RL_KC);
-    const int64_t nksteps = K / 32;
     auto issue_stage = [&](int t) {
         const uint32_t sbase = lds0 + (t % RL_NSTAGE) * RL_STAGE;
         // lanes past the end of the row (last stage of a K that is not a multiple of RL_KC) re-read its start;
@@ -166,7 +168,7 @@ __global__ void __launch_bounds__(RL_THREADS) rows_lora_kernel(const RowsLoraJob
 #pragma unroll
             for (int h = 0; h < NBLK; ++h) {
                 const bf16x8_t x = *(const bf16x8_t*)(st + (h * 8 + (i >> 1)) * RL_PAIRP + (i & 1) * (RL_KC * 2) + wave * 64 + g * 16);
-                acc[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(x, a, acc[h], 0, 0, 0);
+                acc[h] = Num::mfma(x, a, acc[h]);
             }
         }
     }
@@ -186,10 +188,10 @@ __global__ void __launch_bounds__(RL_THREADS) rows_lora_kernel(const RowsLoraJob
 #pragma unroll
             for (int w = 0; w < RL_WAVES; ++w) v += red[w][row][col];
             v *= scaling;
-            Q[mo * 16 + col] = f32_to_bf16_bits(v);
+            Q[mo * 16 + col] = Num::from_f32(v);
             const float vs = qt_row_scale ? v * qt_row_scale[mo] : v;
-            if (Qt) Qt[(int64_t)col * ldqt + mo] = f32_to_bf16_bits(vs);
-            if (job.Qs) job.Qs[mo * 16 + col] = f32_to_bf16_bits(vs);
+            if (Qt) Qt[(int64_t)col * ldqt + mo] = Num::from_f32(vs);
+            if (job.Qs) job.Qs[mo * 16 + col] = Num::from_f32(vs);
         }
     }
 }
@@ -208,6 +210,7 @@ constexpr int XTP_COLS = 4 * XTP_WCOLS;  // columns per workgroup
 // one or two jobs per launch (blockIdx.z): same rows and shapes, different operands / outputs; job j's partials start
 // at partial + j * partial_stride
 struct XtpJob { const uint16_t* X; const uint16_t* Pt; uint16_t* out; int64_t soe, sok, sor; int rank; };   // rank: columns written (<= 16)
+template <typename Num>
 __global__ void __launch_bounds__(XTP_THREADS) xtp_partial_kernel(const XtpJob job0, const XtpJob job1, int64_t ldx,
                                                                   const void* __restrict__ pos, int pos64, int fan_out,
                                                                   int64_t ldpt,
@@ -259,7 +262,7 @@ __global__ void __launch_bounds__(XTP_THREADS) xtp_partial_kernel(const XtpJob j
         for (int t = 0; t < 8; ++t) {
             const float sc = s_scale[t0 + t];   // 0 outside the tile (where Pt may hold anything)
             if (sc == 0.f) pb.h[t] = 0;
-            else if (sc != 1.f) pb.h[t] = f32_to_bf16_bits(bf16_bits_to_f32(pb.h[t]) * sc);
+            else if (sc != 1.f) pb.h[t] = Num::from_f32(Num::to_f32(pb.h[t]) * sc);
         }
         uint32_t w[8][4];   // w[rr][c]: row rr, column pair c
 #pragma unroll
@@ -272,7 +275,7 @@ __global__ void __launch_bounds__(XTP_THREADS) xtp_partial_kernel(const XtpJob j
                 const uint32_t lo = w[2 * qd][j >> 1], hi = w[2 * qd + 1][j >> 1];
                 a.u[qd] = (j & 1) ? ((lo >> 16) | (hi & 0xffff0000u)) : ((lo & 0xffffu) | (hi << 16));
             }
-            acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pb.v, acc[j], 0, 0, 0);
+            acc[j] = Num::mfma(a.v, pb.v, acc[j]);
         }
     };
     uint4 in0[8], in1[8];
@@ -298,6 +301,7 @@ __global__ void __launch_bounds__(XTP_THREADS) xtp_partial_kernel(const XtpJob j
 
 // out[e][k][r] = scale * sum over the expert's partial tiles (ascending), zero for an empty expert.  A thread owns four
 // consecutive rank columns of one k (one 16-byte load per tile, several tiles in flight).
+template <typename Num>
 __global__ void xtp_reduce_kernel(const float* __restrict__ partial, int64_t partial_stride, const XtpJob job0,
                                   const XtpJob job1, const void* __restrict__ offsets, int off64,
                                   int E, int64_t K, float scale)
@@ -335,11 +339,12 @@ __global__ void xtp_reduce_kernel(const float* __restrict__ partial, int64_t par
     }
 #pragma unroll
     for (int q = 0; q < 4; ++q)
-        if (r + q < rank) out[(int64_t)e * soe + k * sok + (r + q) * sor] = f32_to_bf16_bits(s[q] * scale);
+        if (r + q < rank) out[(int64_t)e * soe + k * sok + (r + q) * sor] = Num::from_f32(s[q] * scale);
 }
 
 // Q[m][r] = bf16(scaling * sum_t partial[t][m][r]) (t ascending: a fixed order) and Qt[r][m] likewise.  A thread owns
 // four consecutive rank columns of one row and keeps eight loads in flight.
+template <typename Num>
 __global__ void cc_reduce_kernel(const float* __restrict__ partial0, const float* __restrict__ partial1, int ntiles, int64_t R,
                                  float scaling, uint16_t* __restrict__ Q0, uint16_t* __restrict__ Q1, uint16_t* __restrict__ Qt0,
                                  uint16_t* __restrict__ Qt1, int64_t ldqt)
@@ -369,7 +374,7 @@ __global__ void cc_reduce_kernel(const float* __restrict__ partial0, const float
     }
     uint16_t o[4];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) o[q] = f32_to_bf16_bits(s[q] * scaling);
+    for (int q = 0; q < 4; ++q) o[q] = Num::from_f32(s[q] * scaling);
     *(uint2*)(Q + idx) = make_uint2(o[0] | ((uint32_t)o[1] << 16), o[2] | ((uint32_t)o[3] << 16));
     if (Qt) {
         const int64_t m = idx >> 4;
@@ -382,11 +387,11 @@ __global__ void cc_reduce_kernel(const float* __restrict__ partial0, const float
 }  // namespace
 
 int moe_launch_cc_reduce2(const float* partial, const float* partial2, int ntiles, int64_t R, float scaling, void* Q, void* Q2,
-                          void* Qt, void* Qt2, int64_t ldqt, hipStream_t stream)
+                          void* Qt, void* Qt2, int64_t ldqt, hipStream_t stream, int f16)
 {
     if (R == 0) return MOE_OK;
     const bool two = partial2 != nullptr;
-    hipLaunchKernelGGL(cc_reduce_kernel, dim3((unsigned)((R * 4 + 255) / 256), two ? 2u : 1u), dim3(256), 0, stream, partial, partial2,
+    hipLaunchKernelGGL(f16 ? cc_reduce_kernel<NumF16> : cc_reduce_kernel<NumBf16>, dim3((unsigned)((R * 4 + 255) / 256), two ? 2u : 1u), dim3(256), 0, stream, partial, partial2,
                        ntiles, R, scaling, (uint16_t*)Q, (uint16_t*)Q2, (uint16_t*)Qt, (uint16_t*)Qt2, ldqt);
     return moe_launch_status();
 }
@@ -395,10 +400,11 @@ int moe_launch_pack_lora(const void* src, int64_t se, int64_t sk, int64_t sr, vo
                          int transpose, hipStream_t stream)
 {
     if (rank < 1 || rank > 16) return MOE_ERR_UNSUPPORTED;
-    const int64_t total = (int64_t)E * K * 16;
+    const int64_t Kimg = transpose ? (K + 31) / 32 * 32 : K;
+    const int64_t total = (int64_t)E * Kimg * 16;
     if (total == 0) return MOE_OK;
     hipLaunchKernelGGL(pack_lora_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
-                       (const uint16_t*)src, se, sk, sr, (uint16_t*)dst, K, rank, transpose, total);
+                       (const uint16_t*)src, se, sk, sr, (uint16_t*)dst, K, Kimg, rank, transpose, total);
     return moe_launch_status();
 }
 
@@ -422,36 +428,34 @@ int moe_launch_pack_lora_batch(const MoePackBatch& jobs, hipStream_t stream)
 int moe_launch_rows_lora2(const void* X, const void* X2, int64_t ldx, const void* At, const void* At2, void* Q, void* Q2,
                           void* Qt, void* Qt2, int64_t ldqt, const void* pos, int pos64, const void* offsets, int off64,
                           int E, int64_t R, int64_t K, int fan_out, int x_grouped, float scaling,
-                          const float* qt_row_scale, hipStream_t stream, void* q_scaled)
+                          const float* qt_row_scale, hipStream_t stream, void* q_scaled, int f16)
 {
     if (R == 0) return MOE_OK;
     const bool two = X2 != nullptr;
-    if (K % 32 != 0 || ldx % 8 != 0 || ((uintptr_t)X % 16) != 0 || ((uintptr_t)At % 16) != 0 ||
+    if (K % 8 != 0 || ldx % 8 != 0 || ((uintptr_t)X % 16) != 0 || ((uintptr_t)At % 16) != 0 ||
         (two && (((uintptr_t)X2 % 16) != 0 || ((uintptr_t)At2 % 16) != 0)))
         return MOE_ERR_UNSUPPORTED;
-    static std::atomic<bool> attr_set{false};   // forward and backward may call from different host threads
-    if (!attr_set) {
-        if (hipFuncSetAttribute((const void*)rows_lora_kernel<32>, hipFuncAttributeMaxDynamicSharedMemorySize, rl_lds(32)) != hipSuccess ||
-            hipFuncSetAttribute((const void*)rows_lora_kernel<16>, hipFuncAttributeMaxDynamicSharedMemorySize, rl_lds(16)) != hipSuccess)
+    static std::atomic<bool> attr_set[MOE_MAX_DEVICES];   // per device; forward and backward may call from different host threads
+    const int dev = moe_current_device();
+    if (!attr_set[dev]) {
+        if (hipFuncSetAttribute((const void*)rows_lora_kernel<32, NumBf16>, hipFuncAttributeMaxDynamicSharedMemorySize, rl_lds(32)) != hipSuccess ||
+            hipFuncSetAttribute((const void*)rows_lora_kernel<16, NumBf16>, hipFuncAttributeMaxDynamicSharedMemorySize, rl_lds(16)) != hipSuccess ||
+            hipFuncSetAttribute((const void*)rows_lora_kernel<32, NumF16>, hipFuncAttributeMaxDynamicSharedMemorySize, rl_lds(32)) != hipSuccess ||
+            hipFuncSetAttribute((const void*)rows_lora_kernel<16, NumF16>, hipFuncAttributeMaxDynamicSharedMemorySize, rl_lds(16)) != hipSuccess)
             return MOE_ERR_LAUNCH;
-        attr_set = true;
+        attr_set[dev] = true;
     }
     const RowsLoraJob j0 = {(const uint16_t*)X, (const uint16_t*)At, (uint16_t*)Q, (uint16_t*)Qt, (uint16_t*)q_scaled};
     const RowsLoraJob j1 = {(const uint16_t*)X2, (const uint16_t*)At2, (uint16_t*)Q2, (uint16_t*)Qt2, nullptr};
     // 32-row tiles halve the adapter traffic, but two workgroups fit a compute unit: use them when the launch has
     // about that many, otherwise 16-row tiles (three fit)
-    static std::atomic<int> cus{0};
-    if (cus == 0) {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1) n = 256;
-        cus = n;
-    }
+    const int cus = moe_device_cus();
     const int64_t tiles32 = (R / 32 + E) * (two ? 2 : 1);
     if (tiles32 >= 3 * (int64_t)cus / 2) {
-        hipLaunchKernelGGL(rows_lora_kernel<32>, dim3((unsigned)(R / 32 + E), two ? 2u : 1u), dim3(RL_THREADS), rl_lds(32), stream, j0, j1,
+        hipLaunchKernelGGL((f16 ? rows_lora_kernel<32, NumF16> : rows_lora_kernel<32, NumBf16>), dim3((unsigned)(R / 32 + E), two ? 2u : 1u), dim3(RL_THREADS), rl_lds(32), stream, j0, j1,
                            ldx, ldqt, pos, pos64, offsets, off64, E, K, fan_out, x_grouped, scaling, qt_row_scale);
     } else {
-        hipLaunchKernelGGL(rows_lora_kernel<16>, dim3((unsigned)(R / 16 + E), two ? 2u : 1u), dim3(RL_THREADS), rl_lds(16), stream, j0, j1,
+        hipLaunchKernelGGL((f16 ? rows_lora_kernel<16, NumF16> : rows_lora_kernel<16, NumBf16>), dim3((unsigned)(R / 16 + E), two ? 2u : 1u), dim3(RL_THREADS), rl_lds(16), stream, j0, j1,
                            ldx, ldqt, pos, pos64, offsets, off64, E, K, fan_out, x_grouped, scaling, qt_row_scale);
     }
     return moe_launch_status();
@@ -459,10 +463,10 @@ int moe_launch_rows_lora2(const void* X, const void* X2, int64_t ldx, const void
 
 int moe_launch_rows_lora(const void* X, int64_t ldx, const void* At, void* Q, void* Qt, int64_t ldqt, const void* pos,
                          int pos64, const void* offsets, int off64, int E, int64_t R, int64_t K, int fan_out,
-                         int x_grouped, float scaling, const float* qt_row_scale, hipStream_t stream)
+                         int x_grouped, float scaling, const float* qt_row_scale, hipStream_t stream, int f16)
 {
     return moe_launch_rows_lora2(X, nullptr, ldx, At, nullptr, Q, nullptr, Qt, nullptr, ldqt, pos, pos64, offsets, off64, E, R,
-                                 K, fan_out, x_grouped, scaling, qt_row_scale, stream);
+                                 K, fan_out, x_grouped, scaling, qt_row_scale, stream, nullptr, f16);
 }
 
 size_t moe_xtp_workspace_bytes(int64_t R, int E, int64_t K)
@@ -473,7 +477,7 @@ size_t moe_xtp_workspace_bytes(int64_t R, int E, int64_t K)
 int moe_launch_xtp2(const void* X, const void* X2, int64_t ldx, const void* pos, int pos64, int fan_out, const void* Pt,
                     const void* Pt2, int64_t ldpt, const float* p_row_scale, void* out, void* out2, const int64_t* so,
                     const int64_t* so2, int rank, int rank2, const void* offsets, int off64, int E, int64_t R, int64_t K,
-                    float scale, void* workspace, size_t workspace_bytes, hipStream_t stream)
+                    float scale, void* workspace, size_t workspace_bytes, hipStream_t stream, int f16)
 {
     if (E == 0 || K == 0) return MOE_OK;
     const bool two = X2 != nullptr;
@@ -489,18 +493,18 @@ int moe_launch_xtp2(const void* X, const void* X2, int64_t ldx, const void* pos,
     const int64_t pstride = (int64_t)(one / sizeof(float));
     if (R > 0) {
         dim3 grid((unsigned)((K + XTP_COLS - 1) / XTP_COLS), (unsigned)tiles, two ? 2u : 1u);
-        hipLaunchKernelGGL(xtp_partial_kernel, grid, dim3(XTP_THREADS), 0, stream, j0, j1, ldx, pos, pos64, fan_out, ldpt,
+        hipLaunchKernelGGL(f16 ? xtp_partial_kernel<NumF16> : xtp_partial_kernel<NumBf16>, grid, dim3(XTP_THREADS), 0, stream, j0, j1, ldx, pos, pos64, fan_out, ldpt,
                            p_row_scale, (float*)workspace, pstride, offsets, off64, E, R, K);
     }
     dim3 rgrid((unsigned)((K * 4 + 255) / 256), (unsigned)E, two ? 2u : 1u);
-    hipLaunchKernelGGL(xtp_reduce_kernel, rgrid, dim3(256), 0, stream, (const float*)workspace, pstride, j0, j1, offsets,
+    hipLaunchKernelGGL(f16 ? xtp_reduce_kernel<NumF16> : xtp_reduce_kernel<NumBf16>, rgrid, dim3(256), 0, stream, (const float*)workspace, pstride, j0, j1, offsets,
                        off64, E, K, scale);
     return moe_launch_status();
 }
 
 int moe_launch_xtp_reduce2(const float* partial, const float* partial2, void* out, void* out2, const int64_t* so,
                            const int64_t* so2, int rank, int rank2, const void* offsets, int off64, int E, int64_t K,
-                           float scale, hipStream_t stream)
+                           float scale, hipStream_t stream, int f16)
 {
     if (E == 0 || K == 0) return MOE_OK;
     const bool two = partial2 != nullptr;
@@ -508,7 +512,7 @@ int moe_launch_xtp_reduce2(const float* partial, const float* partial2, void* ou
     const XtpJob j0 = {nullptr, nullptr, (uint16_t*)out, so[0], so[1], so[2], rank};
     const XtpJob j1 = two ? XtpJob{nullptr, nullptr, (uint16_t*)out2, so2[0], so2[1], so2[2], rank2} : j0;
     dim3 rgrid((unsigned)((K * 4 + 255) / 256), (unsigned)E, two ? 2u : 1u);
-    hipLaunchKernelGGL(xtp_reduce_kernel, rgrid, dim3(256), 0, stream, partial, two ? (int64_t)(partial2 - partial) : 0, j0, j1,
+    hipLaunchKernelGGL(f16 ? xtp_reduce_kernel<NumF16> : xtp_reduce_kernel<NumBf16>, rgrid, dim3(256), 0, stream, partial, two ? (int64_t)(partial2 - partial) : 0, j0, j1,
                        offsets, off64, E, K, scale);
     return moe_launch_status();
 }
@@ -516,9 +520,9 @@ int moe_launch_xtp_reduce2(const float* partial, const float* partial2, void* ou
 int moe_launch_xtp(const void* X, int64_t ldx, const void* pos, int pos64, int fan_out, const void* Pt, int64_t ldpt,
                    const float* p_row_scale, void* out, int64_t soe, int64_t sok, int64_t sor, int rank,
                    const void* offsets, int off64, int E, int64_t R, int64_t K, float scale, void* workspace,
-                   size_t workspace_bytes, hipStream_t stream)
+                   size_t workspace_bytes, hipStream_t stream, int f16)
 {
     const int64_t so[3] = {soe, sok, sor};
     return moe_launch_xtp2(X, nullptr, ldx, pos, pos64, fan_out, Pt, nullptr, ldpt, p_row_scale, out, nullptr, so, nullptr, rank,
-                           0, offsets, off64, E, R, K, scale, workspace, workspace_bytes, stream);
+                           0, offsets, off64, E, R, K, scale, workspace, workspace_bytes, stream, f16);
 }

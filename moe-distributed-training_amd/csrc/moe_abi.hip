@@ -64,7 +64,7 @@ inline bool aligned16(const void* p) { return ((uintptr_t)p % 16) == 0; }
 #define TRY(expr) do { int _s = (expr); if (_s != MOE_OK) return _s; } while (0)
 
 // sizes of the packed adapter images and low-rank interims
-inline size_t pack_bytes(int E, int64_t K) { return al((size_t)E * 16 * (size_t)K * 2); }
+inline size_t pack_bytes(int E, int64_t K) { return al((size_t)E * 16 * (size_t)((K + 31) / 32 * 32) * 2); }   // fragment-order images cover K rounded up to 32
 inline size_t q_bytes(int64_t R) { return al((size_t)pad_rows(R) * 16 * 2); }
 
 }  // namespace
@@ -209,6 +209,8 @@ int moe_padded_block_indices(const void* offsets, int off64, int E, int block_m,
     return moe_launch_padded_blocks(offsets, off64, E, block_m, padded_blocks, out64, cap, num_padded, S(stream));
 }
 
+int64_t moe_gemm_debug_launch_count(void) { return moe_gemm_mfma_launch_count(); }
+
 int64_t moe_gemm_debug_plan_blocks(int64_t R, int E, int64_t N, int pair) { return moe_gemm_plan_blocks(R, E, N, pair); }
 
 int moe_gemm_debug_plan(const void* offsets, int off64, int E, int64_t R, int64_t K, int64_t N, int pair, int nseg,
@@ -239,17 +241,19 @@ int moe_scatter2scatter(const void* X, int64_t sxm, int64_t sxk, const void* W, 
     if (A && rank < 1) return MOE_ERR_BAD_ARG;
     if (R == 0) return MOE_OK;
 
-    // matrix-core path: bf16, unit inner strides, weights either K-contiguous (NT) or N-contiguous (NN)
+    // matrix-core path: bf16 or fp16, unit inner strides, weights either K-contiguous (NT) or N-contiguous (NN)
     const bool nt = (swk == 1), nn = (swn == 1) && !nt;
-    if (dtype == MOE_BF16 && sxk == 1 && syn == 1 && (nt || nn) && (!A || rank <= 16 * MOE_MAX_SLABS)) {
+    const bool two_byte = dtype == MOE_BF16 || dtype == MOE_F16;
+    const int f16 = dtype == MOE_F16;
+    if (two_byte && sxk == 1 && syn == 1 && (nt || nn) && (!A || rank <= 16 * MOE_MAX_SLABS)) {
         MoeGemmParams p = {};
         p.X[0] = (const uint16_t*)X; p.ldx = sxm; p.nseg = 1;
         p.W[0] = (const uint16_t*)W; p.swe = swe; p.ldw = nt ? swn : swk; p.nn = nn ? 1 : 0;
         p.Y[0] = (uint16_t*)Y; p.ldy = sym;
         p.pos = pos; p.pos64 = pos64; p.offsets = offsets; p.off64 = off64;
         p.E = E; p.K = K; p.N = N; p.fan_out = fan_out; p.x_grouped = x_grouped; p.y_grouped = y_grouped;
-        p.epi = MOE_EPI_STORE;
-        bool ok = moe_gemm_mfma_supported(p, R) && (!A || (K % 32 == 0));
+        p.epi = MOE_EPI_STORE; p.f16 = f16;
+        bool ok = moe_gemm_mfma_supported(p, R);
         if (ok) {
             if (workspace_bytes < moe_scatter2scatter_workspace_bytes(R, E, K, N, A ? rank : 0) || !workspace)
                 return MOE_ERR_WORKSPACE;
@@ -271,7 +275,7 @@ int moe_scatter2scatter(const void* X, int64_t sxm, int64_t sxk, const void* W, 
                 for (int hf = 0; hf < nh; hf += 2)   // two products over the same rows per launch
                     TRY(moe_launch_rows_lora2(X, hf + 1 < nh ? X : nullptr, sxm, At[hf], hf + 1 < nh ? At[hf + 1] : nullptr, Q[hf],
                                               hf + 1 < nh ? Q[hf + 1] : nullptr, nullptr, nullptr, 0, pos, pos64, offsets, off64, E, R, K,
-                                              fan_out, x_grouped, scaling, nullptr, S(stream)));
+                                              fan_out, x_grouped, scaling, nullptr, S(stream), nullptr, f16));
                 p.nslab = nh; p.slab_mode = 0;
             }
             return moe_launch_gemm_mfma(p, R, S(stream));
@@ -286,7 +290,7 @@ int moe_scatter2scatter(const void* X, int64_t sxm, int64_t sxk, const void* W, 
 static inline bool bwd_ab_fast(int64_t K, int64_t N, int rank, int dtype, int64_t sdm, int64_t sdn, int64_t sxm,
                                int64_t sxk, const void* DY, const void* X)
 {
-    return dtype == MOE_BF16 && rank >= 1 && sdn == 1 && sxk == 1 && K % 32 == 0 && N % 32 == 0 && sdm % 8 == 0 &&
+    return (dtype == MOE_BF16 || dtype == MOE_F16) && rank >= 1 && sdn == 1 && sxk == 1 && K % 32 == 0 && N % 32 == 0 && sdm % 8 == 0 &&
            sxm % 8 == 0 && aligned16(DY) && aligned16(X);
 }
 
@@ -320,6 +324,7 @@ int moe_group_bwd_ab(const void* DY, int64_t sdm, int64_t sdn, const void* X, in
         const size_t xb = moe_xtp_workspace_bytes(R, E, mx);
         void* xw = ws.take(xb);
         if (!xw) return MOE_ERR_WORKSPACE;
+        const int f16 = dtype == MOE_F16;
         // column r of dA depends only on row r of B and row r of dB only on column r of A, so a rank above 16 is
         // worked through in independent chunks of 16 rank columns
         for (int r0 = 0; r0 < rank; r0 += 16) {
@@ -330,12 +335,12 @@ int moe_group_bwd_ab(const void* DY, int64_t sdm, int64_t sdn, const void* X, in
             uint16_t* DBc = (uint16_t*)DB + r0 * sdbr;
             TRY(moe_launch_pack_lora(Ac, sae, sak, sar, At, E, K, rk, 1, S(stream)));
             TRY(moe_launch_pack_lora(Bc, sbe, sbn, sbr, Bt, E, N, rk, 1, S(stream)));
-            TRY(moe_launch_rows_lora(X, sxm, At, Q, Qt, ldt, nullptr, 0, offsets, off64, E, R, K, 1, 1, scaling, nullptr, S(stream)));
-            TRY(moe_launch_rows_lora(DY, sdm, Bt, P, Pt, ldt, nullptr, 0, offsets, off64, E, R, N, 1, 1, scaling, nullptr, S(stream)));
+            TRY(moe_launch_rows_lora(X, sxm, At, Q, Qt, ldt, nullptr, 0, offsets, off64, E, R, K, 1, 1, scaling, nullptr, S(stream), f16));
+            TRY(moe_launch_rows_lora(DY, sdm, Bt, P, Pt, ldt, nullptr, 0, offsets, off64, E, R, N, 1, 1, scaling, nullptr, S(stream), f16));
             TRY(moe_launch_xtp(X, sxm, nullptr, 0, 1, Pt, ldt, nullptr, DAc, sdae, sdak, sdar, rk, offsets, off64, E, R, K,
-                               1.f, xw, xb, S(stream)));
+                               1.f, xw, xb, S(stream), f16));
             TRY(moe_launch_xtp(DY, sdm, nullptr, 0, 1, Qt, ldt, nullptr, DBc, sdbe, sdbn, sdbr, rk, offsets, off64, E, R, N,
-                               1.f, xw, xb, S(stream)));
+                               1.f, xw, xb, S(stream), f16));
         }
         return MOE_OK;
     }
@@ -359,8 +364,9 @@ int moe_group_bwd_w(const void* DY, int64_t sdm, int64_t sdn, const void* X, int
 {
     if (!DY || !X || !DW || !offsets || E < 1 || R < 0 || K < 0 || N < 0) return MOE_ERR_BAD_ARG;
     if (K == 0 || N == 0) return MOE_OK;
-    if (dtype == MOE_BF16 && sdn == 1 && sxk == 1 && swn == 1) {
+    if ((dtype == MOE_BF16 || dtype == MOE_F16) && sdn == 1 && sxk == 1 && swn == 1) {
         MoeXtyParams p = {};
+        p.f16 = dtype == MOE_F16;
         p.X = (const uint16_t*)X; p.ldx = sxm;
         p.DY = (const uint16_t*)DY; p.ldy = sdm;
         p.DW = (uint16_t*)DW; p.swe = swe; p.ldw = swk;
@@ -420,8 +426,6 @@ int moe_swiglu_bwd(const void* gate, const void* up, const void* dh, void* dgate
 
 // ---------------------------------------------------------------------------------------------------------
 // fused expert MLP
-// A row pitch that is a multiple of 4 KiB sends the same K chunk of every row to the same few L2 channels; operands
-// we are free to re-pitch (activations) are copied once to rows of d + 64 elements.
 static inline size_t sk_bytes_mlp(int64_t R, int E, int64_t d, int64_t f)
 {
     const size_t a = moe_gemm_sk_bytes(R, E, d), b = moe_gemm_sk_bytes(R, E, f);
@@ -453,17 +457,19 @@ static bool mlp_shapes_ok(int64_t d, int64_t f, int64_t ldx, int rank, const voi
 static bool mlp_sizes_ok(int64_t gathered_rows, int64_t ld_gathered, int64_t d, int64_t f)
 {
     const int64_t g4 = (int64_t)1 << 32;
-    return (gathered_rows * ld_gathered + d) * 2 < g4 && (f * d + d) * 2 < g4 && (256 * f + f) * 2 < g4 / 2 && (256 * (d + 64) + d) * 2 < g4 / 2;
+    return (gathered_rows * ld_gathered + d) * 2 < g4 && (f * d + d) * 2 < g4 && (256 * f + f) * 2 < g4 / 2 && (256 * d + d) * 2 < g4 / 2;
 }
 
 int moe_mlp_fwd(const void* x, int64_t ldx, const void* w1, const void* w3, const void* w2, const void* const* lora,
                 const int64_t* ls, int rank, float scaling, void* gate, void* up, void* h, void* y, int64_t ldy,
                 const void* pos, int pos64, const void* offsets, int off64, int E, int64_t R, int64_t d, int64_t f,
-                int fan_out, int y_grouped, void* saved, void* workspace, size_t workspace_bytes, void* stream)
+                int fan_out, int y_grouped, int dtype, void* saved, void* workspace, size_t workspace_bytes, void* stream)
 {
     if (!x || !w1 || !w3 || !w2 || !h || !y || !pos || !offsets || E < 1 || fan_out < 1) return MOE_ERR_BAD_ARG;
     const bool has_lora = lora && lora[0];
     if (has_lora && (!ls || !saved || rank < 1)) return MOE_ERR_BAD_ARG;
+    if (dtype != MOE_BF16 && dtype != MOE_F16) return MOE_ERR_UNSUPPORTED;
+    const int f16 = dtype == MOE_F16;
     if (!mlp_shapes_ok(d, f, ldx, has_lora ? rank : 0, w1, w3, w2, x)) return MOE_ERR_UNSUPPORTED;
     if (!mlp_sizes_ok(R / fan_out, ldx, d, f)) return MOE_ERR_UNSUPPORTED;
     if (R == 0) return MOE_OK;
@@ -511,7 +517,7 @@ int moe_mlp_fwd(const void* x, int64_t ldx, const void* w1, const void* w3, cons
         { TIMED("fwd.rows_lora_x");
         for (int c = 0; c < C; ++c)
             TRY(moe_launch_rows_lora2(x, x, ldx, At1[c], At3[c], svp(0, c), svp(1, c), svp(3, c), svp(4, c), ldt, pos, pos64, offsets,
-                                      off64, E, R, d, fan_out, 0, scaling, nullptr, st)); }
+                                      off64, E, R, d, fan_out, 0, scaling, nullptr, st, nullptr, f16)); }
     }
     {
         MoeGemmParams p = {};
@@ -526,7 +532,7 @@ int moe_mlp_fwd(const void* x, int64_t ldx, const void* w1, const void* w3, cons
         }
         p.Y[0] = (uint16_t*)h; p.Y[1] = (uint16_t*)gate; p.Y[2] = (uint16_t*)up; p.ldy = f;
         p.pos = pos; p.pos64 = pos64; p.offsets = offsets; p.off64 = off64;
-        p.E = E; p.K = d; p.N = f; p.fan_out = fan_out; p.x_grouped = 0; p.y_grouped = 1; p.epi = MOE_EPI_SWIGLU;
+        p.E = E; p.K = d; p.N = f; p.fan_out = fan_out; p.x_grouped = 0; p.y_grouped = 1; p.epi = MOE_EPI_SWIGLU; p.f16 = f16;
         if (fuse_q2) {   // Q2 = h A2 (the w2 GEMM's low-rank operand) as per-column-tile partials from the epilogue
             p.epi = MOE_EPI_SWIGLU_FUSED;
             p.CB[0] = (const uint16_t*)At2c[0]; p.CCP[0] = ccw; p.ncc = 1; p.cc_rows = R;
@@ -540,10 +546,10 @@ int moe_mlp_fwd(const void* x, int64_t ldx, const void* w1, const void* w3, cons
     if (has_lora) {
         TIMED("fwd.rows_lora_h");
         if (fuse_q2)   // the products over each column tile came out of the pair GEMM's epilogue: add the tiles, scale, round
-            TRY(moe_launch_cc_reduce2(ccw, nullptr, (int)((f + 127) / 128), R, scaling, svp(2, 0), nullptr, svp(5, 0), nullptr, ldt, st));
+            TRY(moe_launch_cc_reduce2(ccw, nullptr, (int)((f + 127) / 128), R, scaling, svp(2, 0), nullptr, svp(5, 0), nullptr, ldt, st, f16));
         else
         TRY(moe_launch_rows_lora2(h, C > 1 ? h : nullptr, f, At2c[0], At2c[1], svp(2, 0), C > 1 ? svp(2, 1) : nullptr, svp(5, 0),
-                                  C > 1 ? svp(5, 1) : nullptr, ldt, nullptr, 0, offsets, off64, E, R, f, 1, 1, scaling, nullptr, st));
+                                  C > 1 ? svp(5, 1) : nullptr, ldt, nullptr, 0, offsets, off64, E, R, f, 1, 1, scaling, nullptr, st, nullptr, f16));
     }
     {
         MoeGemmParams p = {};
@@ -555,7 +561,7 @@ int moe_mlp_fwd(const void* x, int64_t ldx, const void* w1, const void* w3, cons
         }
         p.Y[0] = (uint16_t*)y; p.ldy = ldy;
         p.pos = pos; p.pos64 = pos64; p.offsets = offsets; p.off64 = off64;
-        p.E = E; p.K = f; p.N = d; p.fan_out = 1; p.x_grouped = 1; p.y_grouped = y_grouped; p.epi = MOE_EPI_STORE;
+        p.E = E; p.K = f; p.N = d; p.fan_out = 1; p.x_grouped = 1; p.y_grouped = y_grouped; p.epi = MOE_EPI_STORE; p.f16 = f16;
         moe_gemm_sk_attach(p, skws, R, E, d);
         p.counters_clean = counters_clean;
         if (moe_gemm_max_split(p.epi == MOE_EPI_SWIGLU || p.epi == MOE_EPI_SWIGLU_FUSED) > 1) counters_clean = true;   // zeroed by that launch if they were not, and left zero
@@ -570,12 +576,14 @@ int moe_mlp_bwd(const void* dy, int64_t lddy, int dy_grouped, int dy_fan_out, co
                 const int64_t* ls, void* const* lg, const int64_t* gs, int rank, float scaling, const void* gate,
                 const void* up, const void* h, void* dgate, void* dup, void* dx_rows, int64_t lddx, int dx_grouped,
                 const void* pos, int pos64, const void* offsets, int off64, int E, int64_t R, int64_t d, int64_t f,
-                int fan_out, const void* saved, void* workspace, size_t workspace_bytes, void* stream)
+                int fan_out, int dtype, const void* saved, void* workspace, size_t workspace_bytes, void* stream)
 {
     if (!dy || !x || !w1 || !w3 || !w2 || !gate || !up || !h || !dgate || !dup || !dx_rows || !pos || !offsets)
         return MOE_ERR_BAD_ARG;
     const bool has_lora = lora && lora[0];
     if (has_lora && (!ls || !lg || !gs || !saved || rank < 1)) return MOE_ERR_BAD_ARG;
+    if (dtype != MOE_BF16 && dtype != MOE_F16) return MOE_ERR_UNSUPPORTED;
+    const int f16 = dtype == MOE_F16;
     if (!mlp_shapes_ok(d, f, ldx, has_lora ? rank : 0, w1, w3, w2, x) || lddy % 8 != 0 || !aligned16(dy))
         return MOE_ERR_UNSUPPORTED;
     if (dy_fan_out < 1 || fan_out < 1) return MOE_ERR_BAD_ARG;
@@ -640,7 +648,7 @@ int moe_mlp_bwd(const void* dy, int64_t lddy, int dy_grouped, int dy_fan_out, co
         TIMED("bwd.rows_lora_dy");
         TRY(moe_launch_rows_lora2(dy, C > 1 ? dy : nullptr, lddy, bt2[0], bt2[1], pqp(0, 0), C > 1 ? pqp(0, 1) : nullptr, pqp(3, 0),
                                   C > 1 ? pqp(3, 1) : nullptr, ldt, pos, pos64, offsets, off64, E, R, d, dy_fan_out, dy_grouped, scaling,
-                                  row_scale, st, p2s));
+                                  row_scale, st, p2s, f16));
     }
     {
         MoeGemmParams p = {};
@@ -654,7 +662,7 @@ int moe_mlp_bwd(const void* dy, int64_t lddy, int dy_grouped, int dy_fan_out, co
         p.H1 = (const uint16_t*)gate; p.H3 = (const uint16_t*)up; p.ldh = f; p.row_scale = row_scale;
         p.pos = pos; p.pos64 = pos64; p.offsets = offsets; p.off64 = off64;
         p.E = E; p.K = d; p.N = f; p.fan_out = dy_fan_out; p.x_grouped = dy_grouped; p.y_grouped = 1;
-        p.epi = MOE_EPI_SWIGLU_BWD;
+        p.epi = MOE_EPI_SWIGLU_BWD; p.f16 = f16;
         if (fuse_rc) {   // dB1 = Q1^T dgate, dB3 = Q3^T dup, dA2 = h^T (row_scale P2) as per-row-tile partials from the epilogue
             const size_t one = moe_xtp_workspace_bytes(R, E, f);
             p.RC[0] = (const uint16_t*)svp(0, 0); p.RC[1] = (const uint16_t*)svp(1, 0); p.RC[2] = (const uint16_t*)p2s;
@@ -683,24 +691,24 @@ int moe_mlp_bwd(const void* dy, int64_t lddy, int dy_grouped, int dy_fan_out, co
         if (fuse_rc) {   // the sums over each row tile came out of the dh GEMM's epilogue: add the tiles per expert
             const size_t one = moe_xtp_workspace_bytes(R, E, f);
             const float* part = (const float*)xw;
-            TRY(moe_launch_xtp_reduce2(part, part + one / sizeof(float), lg[1], lg[3], sb1, sb3, rank, rank, offsets, off64, E, f, 1.f, st));
-            TRY(moe_launch_xtp_reduce2(part + 2 * (one / sizeof(float)), nullptr, dA2, nullptr, sa2, nullptr, rank, 0, offsets, off64, E, f, 1.f, st));
+            TRY(moe_launch_xtp_reduce2(part, part + one / sizeof(float), lg[1], lg[3], sb1, sb3, rank, rank, offsets, off64, E, f, 1.f, st, f16));
+            TRY(moe_launch_xtp_reduce2(part + 2 * (one / sizeof(float)), nullptr, dA2, nullptr, sa2, nullptr, rank, 0, offsets, off64, E, f, 1.f, st, f16));
         } else
         TRY(moe_launch_xtp2(h, C > 1 ? h : nullptr, f, nullptr, 0, 1, pqp(3, 0), C > 1 ? pqp(3, 1) : nullptr, ldt, nullptr, dA2,
                             C > 1 ? dA2 + 16 * gs[14] : nullptr, sa2, sa2, rank < 16 ? rank : 16, C > 1 ? rank - 16 : 0, offsets, off64, E, R, f,
-                            1.f, xw, xb, st));
+                            1.f, xw, xb, st, f16));
         TRY(moe_launch_xtp2(dy, C > 1 ? dy : nullptr, lddy, dy_grouped ? nullptr : pos, pos64, dy_fan_out, svp(5, 0),
                             C > 1 ? svp(5, 1) : nullptr, ldt, row_scale, dB2, C > 1 ? dB2 + 16 * gs[16] : nullptr, sb2, sb2,
-                            rank < 16 ? rank : 16, C > 1 ? rank - 16 : 0, offsets, off64, E, R, d, 1.f, xw, xb, st)); }
+                            rank < 16 ? rank : 16, C > 1 ? rank - 16 : 0, offsets, off64, E, R, d, 1.f, xw, xb, st, f16)); }
         // ---- w1 / w3 backward
         TIMED("bwd.rows_lora_dgate_dup");
         if (fuse_rc) {   // the products over each column tile came out of the dh GEMM's epilogue: add the tiles, scale, round
             const size_t cone = cc_bytes(R, f) / 2 / sizeof(float);
-            TRY(moe_launch_cc_reduce2(ccw, ccw + cone, (int)((f + 255) / 256), R, scaling, pqp(1, 0), pqp(2, 0), pqp(4, 0), pqp(5, 0), ldt, st));
+            TRY(moe_launch_cc_reduce2(ccw, ccw + cone, (int)((f + 255) / 256), R, scaling, pqp(1, 0), pqp(2, 0), pqp(4, 0), pqp(5, 0), ldt, st, f16));
         } else
         for (int c = 0; c < C; ++c)
             TRY(moe_launch_rows_lora2(dgate, dup, f, bt1[c], bt3[c], pqp(1, c), pqp(2, c), pqp(4, c), pqp(5, c), ldt, nullptr, 0, offsets,
-                                      off64, E, R, f, 1, 1, scaling, nullptr, st));
+                                      off64, E, R, f, 1, 1, scaling, nullptr, st, nullptr, f16));
     }
     {
         MoeGemmParams p = {};
@@ -715,7 +723,7 @@ int moe_mlp_bwd(const void* dy, int64_t lddy, int dy_grouped, int dy_fan_out, co
         }
         p.Y[0] = (uint16_t*)dx_rows; p.ldy = lddx;
         p.pos = pos; p.pos64 = pos64; p.offsets = offsets; p.off64 = off64;
-        p.E = E; p.K = f; p.N = d; p.fan_out = 1; p.x_grouped = 1; p.y_grouped = dx_grouped; p.epi = MOE_EPI_STORE;
+        p.E = E; p.K = f; p.N = d; p.fan_out = 1; p.x_grouped = 1; p.y_grouped = dx_grouped; p.epi = MOE_EPI_STORE; p.f16 = f16;
         moe_gemm_sk_attach(p, skws, R, E, d);
         p.counters_clean = counters_clean;
         if (moe_gemm_max_split(p.epi == MOE_EPI_SWIGLU || p.epi == MOE_EPI_SWIGLU_FUSED) > 1) counters_clean = true;   // zeroed by that launch if they were not, and left zero
@@ -730,10 +738,10 @@ int moe_mlp_bwd(const void* dy, int64_t lddy, int dy_grouped, int dy_fan_out, co
         for (int c = 0; c < C; ++c) {
             const int rk = (rank - 16 * c < 16) ? rank - 16 * c : 16;
             TRY(moe_launch_xtp2(x, x, ldx, pos, pos64, fan_out, pqp(4, c), pqp(5, c), ldt, nullptr, (uint16_t*)lg[0] + 16 * c * gs[2],
-                                (uint16_t*)lg[2] + 16 * c * gs[8], sa1, sa3, rk, rk, offsets, off64, E, R, d, 1.f, xw, xb, st));
+                                (uint16_t*)lg[2] + 16 * c * gs[8], sa1, sa3, rk, rk, offsets, off64, E, R, d, 1.f, xw, xb, st, f16));
             if (!fuse_rc)
             TRY(moe_launch_xtp2(dgate, dup, f, nullptr, 0, 1, svp(3, c), svp(4, c), ldt, nullptr, (uint16_t*)lg[1] + 16 * c * gs[4],
-                                (uint16_t*)lg[3] + 16 * c * gs[10], sb1, sb3, rk, rk, offsets, off64, E, R, f, 1.f, xw, xb, st));
+                                (uint16_t*)lg[3] + 16 * c * gs[10], sb1, sb3, rk, rk, offsets, off64, E, R, f, 1.f, xw, xb, st, f16));
         }
     }
     return MOE_OK;

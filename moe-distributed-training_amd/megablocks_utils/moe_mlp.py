@@ -14,7 +14,7 @@ from typing import NamedTuple, Optional, Tuple
 import torch
 import torch.nn as nn
 
-from .._lib import lib, check, is64, ptr, require_gpu, stream_ptr, workspace
+from .._lib import lib, check, dtype_code, is64, ptr, require_gpu, stream_ptr, workspace
 from ..scattermoe_utils.kernels import ops
 from ..scattermoe_utils.parallel_experts import parallel_linear
 from ..scattermoe_utils.parallel_linear_lora import parallel_linear_lora
@@ -59,7 +59,9 @@ class LoraViews(NamedTuple):
 
 
 def _fast_path_ok(x, w1, w2, w3, lora: Optional[LoraViews]) -> bool:
-    if x.dtype != torch.bfloat16 or w1.dtype != torch.bfloat16:
+    if x.dtype not in (torch.bfloat16, torch.float16) or w1.dtype != x.dtype:
+        return False
+    if lora is not None and any(t.dtype != x.dtype for t in lora):
         return False
     E, f, d = w1.shape
     if d % 64 or f % 64 or x.stride(-1) != 1 or x.stride(0) % 8:
@@ -70,7 +72,7 @@ def _fast_path_ok(x, w1, w2, w3, lora: Optional[LoraViews]) -> bool:
         return False
     # gathered activation rows and one expert's matrix are addressed with 32-bit byte offsets (the same check the library
     # makes before it enqueues anything); the number of rows is otherwise not limited
-    if (x.size(0) * (d + 64) + d) * 2 >= 1 << 32 or (f * d + d) * 2 >= 1 << 32:
+    if (x.size(0) * x.stride(0) + d) * 2 >= 1 << 32 or (f * d + d) * 2 >= 1 << 32:
         return False
     return True
 
@@ -107,7 +109,7 @@ def _mlp_fwd(x, w1, w3, w2, lora, scaling, ssi, offsets, fan_out, y_grouped, sav
     lp, ls = (None, None) if lora is None else _lora_arrays(lora)
     check(lib.moe_mlp_fwd(ptr(x), x.stride(0), ptr(w1), ptr(w3), ptr(w2), lp, ls, rank, scaling, ptr(gate), ptr(up),
                           ptr(h), ptr(y), y.stride(0), ptr(ssi), is64(ssi), ptr(offsets), is64(offsets), E, R, d, f,
-                          fan_out, int(y_grouped), ptr(saved), ptr(ws), ws.numel(), stream_ptr(dev)), "moe_mlp_fwd")
+                          fan_out, int(y_grouped), dtype_code(x), ptr(saved), ptr(ws), ws.numel(), stream_ptr(dev)), "moe_mlp_fwd")
     return gate, up, h, y, saved
 
 
@@ -130,7 +132,7 @@ def _mlp_bwd(dy, dy_grouped, dy_fan_out, row_scale, x, w1, w3, w2, lora, scaling
     check(lib.moe_mlp_bwd(ptr(dy), dy.stride(0), int(dy_grouped), dy_fan_out, ptr(row_scale), ptr(x), x.stride(0),
                           ptr(w1), ptr(w3), ptr(w2), lp, ls, gp, gs, rank, scaling, ptr(gate), ptr(up), ptr(h),
                           ptr(dgate), ptr(dup), ptr(dx_rows), dx_rows.stride(0), int(dx_grouped), ptr(ssi), is64(ssi),
-                          ptr(offsets), is64(offsets), E, R, d, f, fan_out, ptr(saved), ptr(ws), ws.numel(),
+                          ptr(offsets), is64(offsets), E, R, d, f, fan_out, dtype_code(x), ptr(saved), ptr(ws), ws.numel(),
                           stream_ptr(dev)), "moe_mlp_bwd")
     return dx_rows, grads, dgate, dup
 

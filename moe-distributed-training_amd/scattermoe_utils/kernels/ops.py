@@ -42,23 +42,29 @@ def flatten_and_sort(expert_idxs: torch.Tensor, num_experts: Optional[int] = Non
     assignments -- the tuple megablocks_utils/config_utils.py:131-132 feeds to the kernels.  Like the ``torch.sort`` it
     stands in for, the sorted ids keep the input's dtype, the positions are int64, and nothing synchronises with the
     host (so the call can be captured into a graph).  The function it replaces has no expert-count argument: without
-    ``num_experts`` the sort runs with the largest count it supports (ids must be below 4096), which costs a few
-    microseconds more than the exact count."""
+    ``num_experts`` the sort runs with the largest count it supports, ``MAX_EXPERTS``, which costs a few microseconds
+    more than the exact count.
+
+    Ids outside ``[0, num_experts)`` (``[0, MAX_EXPERTS)`` without the argument) take no part in the sorted order: the
+    valid assignments fill the front of both outputs and every entry behind them reads ``-1`` (never uninitialised
+    memory), so ``(sorted_expert_idxs < 0).any()`` tells a caller that ids were out of range.  An expert count above
+    ``MAX_EXPERTS`` is refused (``RuntimeError``, from the library's status) before anything is enqueued."""
     dev = require_gpu(expert_idxs)
     flat = expert_idxs.reshape(-1).contiguous()
     if flat.dtype not in (torch.int32, torch.int64):
         flat = flat.to(torch.int64)
     E = MAX_EXPERTS if num_experts is None else int(num_experts)
-    sei, ssi = _sort(flat, E, want_meta=False)[:2]
+    sei, ssi = _sort(flat, E, want_meta=False, sentinel=True)[:2]
     return sei, ssi if ssi.dtype == torch.int64 else ssi.long()
 
 
-def _sort(flat: torch.Tensor, E: int, want_meta: bool = True, block_m: int = BLOCK_M):
-    """Stable counting sort on the device. Returns (sei, ssi, counts, offsets, padded_blocks_buf, num_padded, inv)."""
+def _sort(flat: torch.Tensor, E: int, want_meta: bool = True, block_m: int = BLOCK_M, sentinel: bool = False):
+    """Stable counting sort on the device. Returns (sei, ssi, counts, offsets, padded_blocks_buf, num_padded, inv).
+    ``sentinel``: entries that no valid id lands on (ids outside [0, E) are left out of the order) read -1."""
     dev = flat.device
     R = flat.numel()
-    sei = torch.empty_like(flat)
-    ssi = torch.empty_like(flat)
+    sei = torch.full_like(flat, -1) if sentinel else torch.empty_like(flat)
+    ssi = torch.full_like(flat, -1) if sentinel else torch.empty_like(flat)
     counts = torch.empty(E, dtype=flat.dtype, device=dev) if want_meta else None
     offsets = torch.empty(E, dtype=flat.dtype, device=dev) if want_meta else None
     cap = R // block_m + E

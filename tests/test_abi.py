@@ -31,7 +31,7 @@ def test_library_exports_every_declared_symbol():
     assert set(decls) == set(_lib._SIGNATURES), set(decls) ^ set(_lib._SIGNATURES)
     for name, codes in decls.items():
         assert _lib._SIGNATURES[name][1] == codes, f"binding of {name} disagrees with the header"
-    assert _lib.lib.moe_hip_abi_version() == 1
+    assert _lib.lib.moe_hip_abi_version() == _lib.ABI_VERSION == int(re.search(r"#define\s+MOE_HIP_ABI_VERSION\s+(\d+)", open(os.path.join(ROOT, "include", "moe_hip.h")).read()).group(1))
 
 
 def test_bad_arguments_are_rejected_on_the_host():
@@ -45,8 +45,12 @@ def test_bad_arguments_are_rejected_on_the_host():
     assert lib.moe_group_bwd_ab(None, 1, 1, None, 1, 1, None, 1, 1, 1, None, 1, 1, 1, 4, 1.0, None, 1, 1, 1, None, 1, 1, 1,
                                 None, 0, 2, 8, 16, 16, 0, None, 0, None) == -1
     assert lib.moe_mlp_fwd(None, 1, None, None, None, None, None, 0, 0.0, None, None, None, None, 1, None, 0, None, 0, 2,
-                           8, 64, 64, 1, 0, None, None, 0, None) == -1
+                           8, 64, 64, 1, 0, 0, None, None, 0, None) == -1
     assert lib.moe_sort_workspace_bytes(8192, 8) >= 4 * 8 * 4
+    # the sort's status path: more experts than the counting sort takes (4096) is refused before anything is enqueued
+    # (16: non-null stand-ins that are never dereferenced); this is what flatten_and_sort's RuntimeError comes from
+    assert lib.moe_sort_by_expert(16, 0, 8, 4097, 128, 16, 16, 0, None, None, None, 0, None, None, 16, 1 << 20, None) == -1
+    assert lib.moe_sort_by_expert_static(16, 0, 8, 4097, 128, 16, 16, 0, None, None, None, 0, None, None, None) == -1
     assert lib.moe_mlp_workspace_bytes(8192, 8, 4096, 14336, 16) > 0
 
 
@@ -69,8 +73,8 @@ def test_size_limits_are_checked_before_anything_is_enqueued():
 
     def fwd(R, d, f, fan_out):
         return lib.moe_mlp_fwd(one, d, one, one, one, None, None, 0, 0.0, one, one, one, one, d, one, 0, one, 0, 8,
-                               R, d, f, fan_out, 0, None, None, 0, None)
-    # a gathered x of 4 GiB or more: T * (d + 64) * 2 bytes
+                               R, d, f, fan_out, 0, 0, None, None, 0, None)
+    # a gathered x of 4 GiB or more: T * ldx * 2 bytes
     assert fwd(2 * 600000, 4096, 14336, 2) == -2
     # one expert's matrix of 4 GiB or more
     assert fwd(8192, 65536, 32768, 2) == -2

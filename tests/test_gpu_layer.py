@@ -87,6 +87,40 @@ def test_layer_fwd_bwd_bf16(dev, oracle, T, d, f, E, r):
     assert torch.equal(out2, out) and torch.equal(ei2, ei)
 
 
+@pytest.mark.parametrize("T,d,f,E,r", [(512, 256, 512, 8, 16), (700, 128, 320, 4, 0), (900, 192, 256, 8, 32)])
+def test_layer_fwd_bwd_fp16(dev, oracle, T, d, f, E, r):
+    """The reference's fp16 switch (megablocks_utils/shard_moe_utils.py:29-30,43-44): the whole layer in IEEE half runs the
+    same matrix-core kernels as bf16 (every grouped GEMM launch is counted); fp16 carries 3 more mantissa bits, so the
+    bound is tighter than bf16's."""
+    import moe_distributed_training_amd as moe
+    from moe_distributed_training_amd._lib import lib
+    k, alpha, tol = 2, 32.0, 3e-3
+    x, wg, w1, w2, w3, lora, dout = _make(T, d, f, E, r, torch.float16, seed=T)
+    xo = x.float().requires_grad_(True)
+    lo = None if lora is None else {n: (a.float().requires_grad_(True), b.float().requires_grad_(True)) for n, (a, b) in lora.items()}
+    full = lora is None
+    wo = [w.float().requires_grad_(full) for w in (w1, w2, w3)]
+    ref, aux = oracle.moe_block(xo, wg.float(), wo[0], wo[1], wo[2], k, lo, alpha)
+    ref.backward(dout.float())
+    xg = x.to(dev).requires_grad_(True)
+    lt, views = (None, None) if lora is None else _views(lora, dev)
+    wd = [w.to(dev).requires_grad_(full) for w in (w1, w2, w3)]
+    n0 = lib.moe_gemm_debug_launch_count()
+    out, ew, ei = moe.moe_layer_forward(xg, wg.to(dev), wd[0], wd[1], wd[2], k, views, alpha)
+    out.backward(dout.to(dev))
+    assert lib.moe_gemm_debug_launch_count() - n0 == 4, "pair, h W2, dh and dX GEMMs on the matrix cores"
+    assert out.dtype == torch.float16 and xg.grad.dtype == torch.float16
+    assert torch.equal(ei.cpu().long(), aux["indices"])
+    assert rel(out, ref) < tol and rel(xg.grad, xo.grad) < tol
+    if full:
+        for n, a, b in zip(("w1", "w2", "w3"), wd, wo):
+            check_expert_grads(a.grad, b.grad, f"dW {n}", tol)
+    else:
+        for n in ("w1", "w3", "w2"):
+            check_expert_grads(lt[n][0].grad, lo[n][0].grad, f"dA {n}", tol)
+            check_expert_grads(lt[n][1].grad, lo[n][1].grad, f"dB {n}", tol)
+
+
 @pytest.mark.parametrize("E,k,r", [(96, 4, 16), (16, 8, 16), (80, 3, 0)])
 def test_layer_many_experts_and_wider_top_k(dev, oracle, E, k, r):
     """More than 8 experts (router on the two-launch path), more than 64 (serial group lookup in every grouped kernel),
@@ -321,6 +355,58 @@ def test_mixtral_shape_full_size(dev, oracle):
 
 
 @pytest.mark.slow
+def test_mixtral_shape_forward_without_adapters_full_size(dev, oracle):
+    """BASELINE configs[1] exactly: T=4096, d=4096, f=14336, E=8, top-2, near-uniform routing, no adapters, forward
+    only -- the adapter-free gate/up kernel variant and its tile plan at the full size, against the fp32 oracle."""
+    import moe_distributed_training_amd as moe
+    T, d, f, E, k = 4096, 4096, 14336, 8, 2
+    g = torch.Generator(device=dev).manual_seed(1)
+    rn = lambda *s, std=1.0: (torch.randn(*s, generator=g, device=dev) * std).bfloat16()
+    x, wg = rn(T, d), rn(E, d, std=0.02)
+    w1, w2, w3 = rn(E, f, d, std=0.02), rn(E, f, d, std=0.02), rn(E, f, d, std=0.02)
+    with torch.no_grad():
+        out, ew, ei = moe.moe_layer_forward(x, wg, w1, w2, w3, k, None, 1.0)
+        torch.cuda.synchronize()
+        torch.set_num_threads(16)
+        ref, aux = oracle.moe_block(x.float().cpu(), wg.float().cpu(), w1.float().cpu(), w2.float().cpu(), w3.float().cpu(), k)
+    counts = torch.bincount(aux["indices"].flatten(), minlength=E)
+    assert counts.min() > 0.8 * T * k / E and counts.max() < 1.2 * T * k / E   # near-uniform, as the configuration says
+    flips = int((ei.cpu().long() != aux["indices"]).any(-1).sum())
+    assert flips == 0, f"{flips} tokens routed differently from the fp32 oracle"
+    assert torch.allclose(ew.float().cpu(), aux["weights"], atol=2e-3)
+    assert rel(out, ref) < 1e-2
+
+
+@pytest.mark.slow
+def test_mixtral_shape_full_finetune_full_size(dev, oracle):
+    """Full fine-tuning (no adapters, the stored expert weights take gradients) at the Mixtral shape, T=4096, fwd+bwd:
+    out, dX and dW1 / dW3 / dW2 of every expert (max and RMS on the expert's own scale) against the fp32 oracle."""
+    import moe_distributed_training_amd as moe
+    T, d, f, E, k = 4096, 4096, 14336, 8, 2
+    g = torch.Generator(device=dev).manual_seed(2)
+    rn = lambda *s, std=1.0: (torch.randn(*s, generator=g, device=dev) * std).bfloat16()
+    x, wg = rn(T, d), rn(E, d, std=0.02)
+    wd = [rn(E, f, d, std=0.02).requires_grad_(True) for _ in range(3)]      # w1, w2, w3
+    dout = rn(T, d)
+    xg = x.clone().requires_grad_(True)
+    out, ew, ei = moe.moe_layer_forward(xg, wg, wd[0], wd[1], wd[2], k, None, 1.0)
+    out.backward(dout)
+    torch.cuda.synchronize()
+    torch.set_num_threads(16)
+    xo = x.float().cpu().requires_grad_(True)
+    wo = [w.detach().float().cpu().requires_grad_(True) for w in wd]
+    ref, aux = oracle.moe_block(xo, wg.float().cpu(), wo[0], wo[1], wo[2], k)
+    ref.backward(dout.float().cpu())
+    assert torch.equal(ei.cpu().long(), aux["indices"])
+    assert rel(out, ref) < 1e-2 and rel(xg.grad, xo.grad) < 1e-2
+    for n, a, b in zip(("w1", "w2", "w3"), wd, wo):
+        assert a.grad is not None and a.grad.shape == b.grad.shape
+        check_expert_grads(a.grad, b.grad, f"dW {n}")
+        a.grad = None
+        b.grad = None
+
+
+@pytest.mark.slow
 def test_mixtral_shape_skewed_routing_full_gradients(dev, oracle):
     """BASELINE configs[3]'s routing (Zipf s=1.2 logit offsets: the top expert takes ~40 % of the assignments, the
     last ones are near-empty) at the real d, f with LoRA, T=4096, fwd+bwd: out, dX and all six adapter gradients
@@ -534,10 +620,10 @@ def test_skewed_full_size_properties(dev, oracle):
     assert rel(out[sl], ref) < 1e-2 and rel(dx1[sl], xo.grad) < 1e-2
     # (4) adapter gradients of single experts against the oracle: an expert's dA / dB depend only on the rows routed to
     # it, so the oracle run on those tokens alone (one assignment each, the layer's own routing weight) gives them.  The
-    # smallest group (near-empty) and a mid-sized one; the largest is covered at T=4096 with the same routing law.
+    # smallest group (near-empty), a mid-sized one and the largest (the only group with more than 50 row tiles).
     ewc, eic = ew.float().cpu(), ei.cpu().long()
     order = torch.argsort(counts)
-    for e in (int(order[0]), int(order[E // 2])):
+    for e in (int(order[0]), int(order[E // 2]), int(order[-1])):
         tok, slot = torch.where(eic == e)
         loe = {n: (a.float().cpu().requires_grad_(True), b.float().cpu().requires_grad_(True)) for n, (a, b) in lora.items()}
         refe, _ = oracle.moe_block(x[tok.to(dev)].float().cpu(), None, w1.float().cpu(), w2.float().cpu(), w3.float().cpu(), 1, loe, alpha,

@@ -40,8 +40,11 @@ CASES = [
     # dtype, T, E, k, K, N, r
     (torch.float32, 10, 2, 1, 128, 16, 16),      # the reference's own test shape
     (torch.float32, 300, 4, 2, 100, 36, 4),
-    (torch.float16, 300, 4, 2, 64, 40, 8),
-    (torch.bfloat16, 300, 4, 2, 72, 40, 8),      # K not a multiple of 64 -> generic kernels
+    (torch.float16, 300, 4, 2, 64, 40, 8),       # fp16 on the matrix cores
+    (torch.bfloat16, 300, 4, 2, 72, 40, 8),      # K not a multiple of 64: a partial last K tile, masked loads
+    (torch.float16, 700, 8, 2, 200, 264, 16),    # fp16, three whole K tiles and a partial one, N tail, adapters
+    (torch.bfloat16, 500, 4, 2, 1096, 512, 24),  # split K with a partial last tile, two adapter slabs
+    (torch.bfloat16, 300, 4, 2, 40, 64, 8),      # K below one K tile -> generic kernels
     (torch.bfloat16, 1000, 8, 2, 256, 512, 16),
     (torch.bfloat16, 1500, 8, 2, 512, 264, 16),  # N tail inside a 256-wide tile
     (torch.bfloat16, 700, 3, 2, 1024, 256, 4),   # rank < 16 zero padded
@@ -66,14 +69,21 @@ def test_scatter2scatter_all_row_mappings(dev, oracle, layout, dtype, T, E, k, K
     A = (torch.randn(E, K, r) * 0.05).to(dtype)
     B = (torch.randn(E, r, N) * 0.05).to(dtype)
     seid, ssid = sei.to(dev), ssi.int().to(dev)            # mixed index widths on purpose
+    # which kernel a shape takes: 2-byte types with K >= 64 and K, N multiples of 8 run on the matrix cores (one grouped
+    # GEMM launch per call), everything else on the generic kernels
+    from moe_distributed_training_amd._lib import lib
+    on_matrix_cores = dtype != torch.float32 and K >= 64 and K % 8 == 0 and N % 8 == 0
     for xg, yg in [(False, True), (False, False), (True, False), (True, True)]:
         X = torch.randn(T * k if xg else T, K).to(dtype)
         kk = 1 if xg else k
         s_in = ssi if not xg else ssi
+        n0 = lib.moe_gemm_debug_launch_count()
         y = ops.scatter2scatter_lora(X.to(dev), W.to(dev), A.to(dev), B.to(dev), 32.0, seid, ssid, kk, None, xg, yg)
+        assert lib.moe_gemm_debug_launch_count() - n0 == int(on_matrix_cores)
         yo = oracle.scatter2scatter_lora(X, W, A, B, 32.0, sei, s_in, kk, None, xg, yg)
         assert rel(y, yo) < TOL[dtype], (xg, yg)
         y2 = ops.scatter2scatter(X.to(dev), W.to(dev), seid, ssid, kk, None, xg, yg)
+        assert lib.moe_gemm_debug_launch_count() - n0 == 2 * int(on_matrix_cores)
         yo2 = oracle.scatter2scatter_lora(X, W, None, None, 0.0, sei, s_in, kk, None, xg, yg)
         assert rel(y2, yo2) < TOL[dtype], (xg, yg)
 

@@ -175,6 +175,29 @@ def test_flatten_and_sort_never_synchronises(dev):
         assert torch.equal(sei.cpu(), want_e) and torch.equal(ssi.cpu(), want_p)
 
 
+def test_flatten_and_sort_marks_ids_out_of_range(dev):
+    """Ids the counting sort cannot place (negative, or at / above the expert count -- 4096 without the argument) take no
+    part in the order: the valid entries come first, stably sorted, and everything behind them reads -1 in both outputs,
+    never uninitialised memory; more experts than the sort takes is an error before anything is enqueued."""
+    _, _, ops = _mods()
+    g = torch.Generator().manual_seed(5)
+    for n_exp, limit in ((None, ops.MAX_EXPERTS), (8, 8)):
+        t = torch.randint(0, limit, (3001,), generator=g)
+        bad = torch.randperm(3001, generator=g)[:37]
+        t[bad[:20]] = limit + torch.arange(20)       # too large
+        t[bad[20:]] = -1 - torch.arange(17)          # negative
+        for dt in (torch.int32, torch.int64):
+            sei, ssi = ops.flatten_and_sort(t.to(dt).to(dev), num_experts=n_exp)
+            keep = (t >= 0) & (t < limit)
+            want_e, order = torch.sort(t[keep], stable=True)
+            want_p = torch.where(keep)[0][order]
+            n = int(keep.sum())
+            assert torch.equal(sei.cpu()[:n].long(), want_e) and torch.equal(ssi.cpu()[:n], want_p)
+            assert bool((sei.cpu()[n:] == -1).all()) and bool((ssi.cpu()[n:] == -1).all()) and sei.numel() - n == 37
+    with pytest.raises(RuntimeError, match="bad argument"):
+        ops.flatten_and_sort(torch.zeros(16, dtype=torch.int64, device=dev), num_experts=ops.MAX_EXPERTS + 1)
+
+
 def test_sort_is_deterministic(dev):
     _, router, _ = _mods()
     t = torch.randint(0, 8, (32768,), device=dev, dtype=torch.int32)
