@@ -793,20 +793,10 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
             }
         stage_flush(WTN, p.Y[0], p.ldy, !p.y_grouped, n0 + wn * WTN);
     } else if (EPI_IS_PAIR(EPI)) {
-        // gate = acc[mb][j], up = acc[mb][NBH + j] at identical (row, column) positions; both are rounded to storage
-        // precision first (in place) so that forward and backward see the same values
+        // gate = acc[mb][j], up = acc[mb][NBH + j] at identical (row, column) positions.  Outputs: Y0 = h = silu(gate) * up,
+        // computed from the fp32 accumulators, and optionally Y1 = gate, Y2 = up for the backward pass.  One sweep produces
+        // all three; gate and up wait for their passes already rounded and packed, in half of the accumulators' registers.
         const int64_t ncol0 = n0 + wn * (WTN / 2);
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-            for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-                for (int r = 0; r < 4; r += 2) {
-                    float a_ = acc[mb][nb][r], b_ = acc[mb][nb][r + 1];
-                    Num::round2(a_, b_);
-                    acc[mb][nb][r] = a_;
-                    acc[mb][nb][r + 1] = b_;
-                }
 #pragma unroll
         for (int pass = 0; pass < 3; ++pass) {
             uint16_t* Y = p.Y[pass];
@@ -815,14 +805,25 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
             for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
                 for (int nj = 0; nj < NBH; ++nj) {
-                    float o[4];
+                    if (pass == 0) {
+                        float o[4], g[4], u[4];
 #pragma unroll
-                    for (int t = 0; t < 4; ++t) {
-                        const float g = acc[mb][nj][t];
-                        const float u = acc[mb][NBH + nj][t];
-                        o[t] = pass == 0 ? g * sigmoid_f(g) * u : (pass == 1 ? g : u);
+                        for (int t = 0; t < 4; ++t) {
+                            g[t] = acc[mb][nj][t];
+                            u[t] = acc[mb][NBH + nj][t];
+                            o[t] = g[t] * sigmoid_f(g[t]) * u[t];
+                        }
+                        stage_put(WTN / 2, mb * 16 + mrow, nj * 16 + nq, pack4(o[0], o[1], o[2], o[3]));
+                        const uint2 pg = pack4(g[0], g[1], g[2], g[3]), pu = pack4(u[0], u[1], u[2], u[3]);
+                        acc[mb][nj][0] = __uint_as_float(pg.x); acc[mb][nj][1] = __uint_as_float(pg.y);
+                        acc[mb][NBH + nj][0] = __uint_as_float(pu.x); acc[mb][NBH + nj][1] = __uint_as_float(pu.y);
+                    } else {
+                        const int src = pass == 1 ? nj : NBH + nj;
+                        uint2 v;
+                        v.x = __float_as_uint(acc[mb][src][0]);
+                        v.y = __float_as_uint(acc[mb][src][1]);
+                        stage_put(WTN / 2, mb * 16 + mrow, nj * 16 + nq, v);
                     }
-                    stage_put(WTN / 2, mb * 16 + mrow, nj * 16 + nq, pack4(o[0], o[1], o[2], o[3]));
                 }
             if (EPI == MOE_EPI_SWIGLU_FUSED && pass == 0) {
                 // Fused column contraction (the low-rank interim of the next GEMM): CCP[0][nt][m][r] = sum_n h[m][n] CB[0][e][n][r]
@@ -904,7 +905,8 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
 #pragma unroll
         for (int it = 0; it < PD; ++it) fetch(it, it);
         // ---- fused low-rank products (EPI = MOE_EPI_SWIGLU_BWD_FUSED): while dgate, dup and h = silu(gate) * up (recomputed
-        // here, bit-identical to the forward's h: same operands, same order) pass through LDS, the tile also produces
+        // here from the stored gate / up; the forward's own h came from the unrounded accumulators and differs from it in
+        // the last bit or two) pass through LDS, the tile also produces
         //   row contractions (adapter gradients that sum over the tile's rows m):
         //     RCP[0][mtile][n][r] = sum_m dgate[m][n] RC[0][m][r],  RCP[1] likewise with dup and RC[1],  RCP[2] with h and RC[2]
         //   column contractions (the low-rank interims of the next GEMM, sums over the tile's columns n):

@@ -117,6 +117,55 @@ __global__ void __launch_bounds__(ROW_THREADS) combine_fwd_kernel(const T* __res
     }
 }
 
+// The same sum for whole 16-byte columns and k <= KMAX: the k row numbers and weights of the token are fetched first,
+// then the k rows' loads of a column chunk are all in flight before the first of them is used -- one trip to memory per
+// chunk instead of one per row (rows j >= k re-read row 0 with weight 0).  The summation order is unchanged.
+template <typename T, int KMAX>
+__global__ void __launch_bounds__(ROW_THREADS) combine_fwd_batched_kernel(const T* __restrict__ y, int64_t ldy,
+                                                                          T* __restrict__ out, int64_t ldo,
+                                                                          const void* __restrict__ gates, int gdtype,
+                                                                          const int32_t* __restrict__ inv, int k,
+                                                                          int64_t ncols,
+                                                                          const float* __restrict__ extra_coef,
+                                                                          const T* __restrict__ extra_rows, int64_t lde,
+                                                                          int n_extra)
+{
+    constexpr int N = Vec8<T>::N;
+    const int64_t t = blockIdx.x;
+    const T* rowp[KMAX];
+    float g[KMAX];
+#pragma unroll
+    for (int j = 0; j < KMAX; ++j) {
+        const int64_t idx = t * k + (j < k ? j : 0);
+        const int64_t row = inv ? (int64_t)inv[idx] : idx;
+        rowp[j] = y + row * ldy;
+        g[j] = j < k ? (gates ? load_gate(gates, idx, gdtype) : 1.f) : 0.f;
+    }
+#pragma unroll 2
+    for (int64_t c0 = (int64_t)threadIdx.x * N; c0 < ncols; c0 += (int64_t)ROW_THREADS * N) {
+        uint4 raw[KMAX];
+#pragma unroll
+        for (int j = 0; j < KMAX; ++j) raw[j] = *(const uint4*)(rowp[j] + c0);
+        float acc[N];
+#pragma unroll
+        for (int u = 0; u < N; ++u) acc[u] = 0.f;
+#pragma unroll
+        for (int j = 0; j < KMAX; ++j) {
+            const T* e = (const T*)&raw[j];
+#pragma unroll
+            for (int u = 0; u < N; ++u) acc[u] = fmaf(g[j], Elem<T>::ld(e + u), acc[u]);
+        }
+        for (int e = 0; e < n_extra; ++e) {
+            const float ge = extra_coef[t * n_extra + e];
+            float v[N];
+            load_vec<T>(extra_rows + (int64_t)e * lde + c0, v, true, N);
+#pragma unroll
+            for (int u = 0; u < N; ++u) acc[u] = fmaf(ge, v[u], acc[u]);
+        }
+        store_vec<T>(out + t * ldo + c0, acc, true, N);
+    }
+}
+
 // dgates[t*k+j] = <y[row(t,j)], dout[t]>   (one wave per (t,j))
 template <typename T>
 __global__ void __launch_bounds__(ROW_THREADS) combine_dgates_kernel(const T* __restrict__ y, int64_t ldy,
@@ -260,6 +309,11 @@ int moe_launch_combine_fwd(const void* y, int64_t ldy, void* out, int64_t ldo, c
     if (ntok == 0 || ncols == 0) return MOE_OK;
     MOE_DISPATCH_DTYPE(dtype, {
         const int vo = vec_aligned<T>(y, ldy) && vec_aligned<T>(out, ldo) && (!extra_rows || vec_aligned<T>(extra_rows, lde));
+        if (vo && k >= 1 && k <= 8 && ncols % Vec8<T>::N == 0) {
+            auto kern = k <= 2 ? combine_fwd_batched_kernel<T, 2> : (k <= 4 ? combine_fwd_batched_kernel<T, 4> : combine_fwd_batched_kernel<T, 8>);
+            hipLaunchKernelGGL(kern, dim3((unsigned)ntok), dim3(ROW_THREADS), 0, stream, (const T*)y, ldy, (T*)out, ldo, gates, gdtype,
+                               inv, k, ncols, extra_coef, (const T*)extra_rows, lde, n_extra);
+        } else
         hipLaunchKernelGGL((combine_fwd_kernel<T>), dim3((unsigned)ntok), dim3(ROW_THREADS), 0, stream, (const T*)y,
                            ldy, (T*)out, ldo, gates, gdtype, inv, k, ncols, vo, extra_coef, (const T*)extra_rows, lde,
                            n_extra);
