@@ -57,6 +57,7 @@ constexpr int RC_IMG_BYTES = BM * 16 * 2;                       // 8 KiB per ope
 static_assert(RC_IMG_OFF + RC_MATS * RC_IMG_BYTES <= LDS_BYTES, "row-contraction images fit behind the tables");
 constexpr int NXCD = 8;
 constexpr int INTERLEAVE_MIN_ROUNDS = 8;    // launches with at least this many rounds of tiles deal them to the XCDs in chunks
+constexpr int CONTIGUOUS_MIN_ROUNDS = 4;    // ... and so do launches of fewer rounds than this; those in between give every XCD one contiguous range
 
 // 16 bytes per lane, global -> LDS without passing through VGPRs: lane l's data lands at lds_addr + 16*l.  The source
 // is a raw buffer (base address in a scalar resource descriptor) plus a 32-bit per-lane byte offset plus a scalar byte
@@ -126,7 +127,10 @@ __device__ __forceinline__ WorkItem decode_work_item(const void* offsets, int of
         // tiles go to consecutive XCDs instead -- a chunk still runs side by side on its XCD (its tiles share weight and
         // row tiles in that L2), but every XCD sees every part of the list, which evens out the cheaper tiles of ragged
         // groups (measured: the gate/up launch, 16 rounds, 3 % faster dealt out in chunks, the 9-round launches of a
-        // skewed 16384-token batch 8 %; 2-round launches and evenly sized groups up to 2 % slower).  Measured and
+        // skewed 16384-token batch 8 %).  Launches of two or three rounds are dealt out the same way: over eight routing
+        // draws of 8192 rows their two N-contiguous launches run 1-2 % faster than with contiguous ranges (0.4 % of the
+        // layer's GEMM time on average, 1 % on the default draw, and no slower with evenly sized groups), while the
+        // 7-round launch with the SwiGLU-backward epilogue measured 1.5 % slower dealt out and keeps its ranges.  Measured and
         // dropped for launches of few rounds: XCD ranges cut by the running cost of the tiles (32-row blocks, at
         // least half a tile) instead of by their number -- 4-7 % slower, with either way of splitting the last tiles.
         const int64_t F = (T / ncu) * ncu;
@@ -137,7 +141,8 @@ __device__ __forceinline__ WorkItem decode_work_item(const void* offsets, int of
         const int64_t Fx = F / NXCD;
         const int Sx = (S + NXCD - 1) / NXCD;
         if (q < Fx) {
-            t = (F >= (int64_t)INTERLEAVE_MIN_ROUNDS * ncu) ? ((q / CH) * NXCD + xcd) * CH + q % CH : xcd * Fx + q;
+            const bool deal = F >= (int64_t)INTERLEAVE_MIN_ROUNDS * ncu || F < (int64_t)CONTIGUOUS_MIN_ROUNDS * ncu;
+            t = deal ? ((q / CH) * NXCD + xcd) * CH + q % CH : xcd * Fx + q;
         } else {
             const int64_t j = (int64_t)xcd * Sx + (q - Fx);
             if (q - Fx >= Sx || j >= S) return w;
