@@ -214,8 +214,9 @@ __global__ void gemm_plan_kernel(const void* offsets, int off64, int E, int ntil
     }
 }
 
-// KTAIL: K is not a multiple of the 64-wide K tile (but of 8): the last tile of every K segment is partial, and the loads
-// that would reach past K fetch zeros instead.  A variant of its own so that the loop for whole tiles carries none of it.
+// KTAIL, the general variant (plain epilogue only): K need not be a multiple of the 64-wide K tile (but of 8) -- the last
+// tile of every K segment is then partial, and the loads that would reach past K fetch zeros instead -- and the adapter may
+// have more than MOE_MAX_SLABS slabs.  A variant of its own so that the kernels of the usual shapes carry none of it.
 template <bool NN, int EPI, typename Num, bool KTAIL>
 __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGemmParams p)
 {
@@ -655,7 +656,47 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
     // are read from the LDS image that the main loop fetched as "the tile after the last" (the gate/up launch 1.5 %
     // faster than with the round trip to memory here); three or four come straight from global memory, all fragments
     // requested before the first of them is used, so that the tile pays one memory round trip, not one per fragment.
-    {
+    // More than MOE_MAX_SLABS slabs (an adapter rank above 64; general variant, every slab feeds every column): the slabs
+    // are slab_stride-spaced copies of Q[0] / LB[0] and are worked through two per MFMA step in a loop, each step's
+    // fragments straight from global memory -- one round trip per 32 rank columns, paid only by such ranks.
+    if constexpr (KTAIL) {
+        if (p.nslab > MOE_MAX_SLABS) {
+            const int kc = (lane >> 4) & 1;
+            const bool upper = lane >= 32;
+#pragma unroll 1
+            for (int lo = 0; lo < p.nslab; lo += 2) {
+                const bool has_hi = lo + 1 < p.nslab;
+                const int src = (upper && has_hi) ? lo + 1 : lo;
+                const bool live = !upper || has_hi;
+                const uint16_t* Q = p.Q[0] + (int64_t)src * p.q_slab_stride;
+                const uint16_t* LB = p.LB[0] + (int64_t)src * p.lb_slab_stride + (int64_t)expert * p.N * 16;
+                bf16x8_t ta[MB], tb[NB];
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb) {
+                    int64_t n = n0 + wn * WTN + nb * 16 + (lane & 15);
+                    if (n >= p.N) n = p.N - 1;
+                    bf16x8_t v = {};
+                    if (live) v = *(const bf16x8_t*)(LB + n * 16 + 8 * kc);
+                    tb[nb] = v;
+                }
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb) {
+                    int r = wm * WTM + mb * 16 + (lane & 15);
+                    if (r >= nrows) r = nrows - 1;
+                    bf16x8_t v = {};
+                    if (live) v = *(const bf16x8_t*)(Q + (row0 + r) * 16 + 8 * kc);
+                    ta[mb] = v;
+                }
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb)
+                    if (mb < mb_cnt) {
+#pragma unroll
+                        for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = Num::mfma(tb[nb], ta[mb], acc[mb][nb]);
+                    }
+            }
+        }
+    }
+    if (!KTAIL || p.nslab <= MOE_MAX_SLABS) {
         const int kc = (lane >> 4) & 1;          // which 8 of a slab's 16 k this lane holds
         const bool upper = lane >= 32;
         const int per_group = p.slab_mode == 0 ? p.nslab : p.nslab / 2;   // slabs per column group
@@ -1177,7 +1218,7 @@ template <bool NN, int EPI, typename Num, bool KTAIL> int launch_typed(const Moe
 // the kernel variant for the launch's 16-bit storage type
 template <bool NN, int EPI> int launch_variant(const MoeGemmParams& p, int64_t R, hipStream_t stream)
 {
-    if (p.K % BK != 0) {   // a partial last K tile: the plain epilogue only (the fused layer's shapes are whole tiles)
+    if (p.K % BK != 0 || p.nslab > MOE_MAX_SLABS) {   // a partial last K tile, a rank above 64: the plain epilogue only (the fused layer's shapes are whole tiles, its ranks smaller)
         if constexpr (EPI == MOE_EPI_STORE)
             return p.f16 ? launch_typed<NN, EPI, NumF16, true>(p, R, stream) : launch_typed<NN, EPI, NumBf16, true>(p, R, stream);
         else
@@ -1229,8 +1270,9 @@ bool moe_gemm_mfma_supported(const MoeGemmParams& p, int64_t R)
     if (p.K < BK || p.K % 8 != 0 || p.N % 8 != 0 || p.ldx % 8 != 0 || p.ldw % 8 != 0 || p.swe % 8 != 0) return false;
     if (!al16(p.X[0]) || !al16(p.X[1]) || !al16(p.W[0]) || !al16(p.W[1])) return false;
     for (int i = 0; i < MOE_MAX_SLABS; ++i)
-        if (!al16(p.Q[i]) || !al16(p.LB[i])) return false;
-    if (p.nseg < 1 || p.nseg > 2 || p.nslab < 0 || p.nslab > MOE_MAX_SLABS || (p.slab_mode == 1 && p.nslab % 2 != 0)) return false;
+        if (!al16(p.Q[i]) || !al16(p.LB[i])) return false;   // (slabs beyond these: multiples of 16 bytes from Q[0] / LB[0], checked below)
+    if (p.nseg < 1 || p.nseg > 2 || p.nslab < 0 || (p.slab_mode == 1 && p.nslab % 2 != 0)) return false;
+    if (p.nslab > MOE_MAX_SLABS && (p.epi != MOE_EPI_STORE || p.slab_mode != 0 || p.nslab > MOE_MAX_STRIDED_SLABS || p.q_slab_stride % 8 != 0 || p.lb_slab_stride % 8 != 0)) return false;
     // 32-bit byte offsets: gathered A rows from the start of X (grouped ones from the tile's first row), weights from
     // the start of one expert's matrix, grouped outputs and the saved gate / up from the tile's first row; scattered
     // output rows from the start of Y while Y spans less than 2 GiB, 64-bit addresses beyond (y_wide, set at launch)

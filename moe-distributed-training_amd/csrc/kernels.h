@@ -11,7 +11,8 @@
 #define MOE_EPI_SWIGLU_FUSED 4   // as MOE_EPI_SWIGLU, and the product of h with an adapter factor per column tile (CB[0] -> CCP[0], ncc = 1)
 #define MOE_EPI_SWIGLU_BWD_FUSED 3   // ... and the low-rank products of dgate, dup and h that the adapters' backward needs (RC / CB below)
 
-constexpr int MOE_MAX_SLABS = 4;
+constexpr int MOE_MAX_SLABS = 4;            // slabs given by their own pointers
+constexpr int MOE_MAX_STRIDED_SLABS = 16;   // slabs of a plain-epilogue launch laid out at a fixed stride (adapter rank up to 256)
 
 struct MoeGemmParams {
     const uint16_t* X[2];   // A-operand segments, rows of K bf16, unit k stride
@@ -23,7 +24,9 @@ struct MoeGemmParams {
     int nn;
     const uint16_t* Q[MOE_MAX_SLABS];   // low-rank A-side operands [R][16] bf16 in grouped order (already scaled)
     const uint16_t* LB[MOE_MAX_SLABS];  // low-rank B-side operands [E][N][16] bf16
-    int nslab;              // 0..MOE_MAX_SLABS 16-wide K slabs (a rank-r adapter is ceil(r/16) slabs)
+    int nslab;              // 0..MOE_MAX_SLABS 16-wide K slabs (a rank-r adapter is ceil(r/16) slabs); more (up to MOE_MAX_STRIDED_SLABS, plain
+                            // epilogue, slab_mode 0): slab s is Q[0] + s * q_slab_stride, LB[0] + s * lb_slab_stride
+    int64_t q_slab_stride, lb_slab_stride;   // elements
     int slab_mode;          // 0: every slab feeds every column; 1: the first half of the slabs feeds the gate weight of the SwiGLU pair, the second half the up weight
     uint16_t* Y[3];
     int64_t ldy;

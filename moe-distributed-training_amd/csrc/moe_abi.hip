@@ -245,7 +245,7 @@ int moe_scatter2scatter(const void* X, int64_t sxm, int64_t sxk, const void* W, 
     const bool nt = (swk == 1), nn = (swn == 1) && !nt;
     const bool two_byte = dtype == MOE_BF16 || dtype == MOE_F16;
     const int f16 = dtype == MOE_F16;
-    if (two_byte && sxk == 1 && syn == 1 && (nt || nn) && (!A || rank <= 16 * MOE_MAX_SLABS)) {
+    if (two_byte && sxk == 1 && syn == 1 && (nt || nn) && (!A || rank <= 16 * MOE_MAX_STRIDED_SLABS)) {
         MoeGemmParams p = {};
         p.X[0] = (const uint16_t*)X; p.ldx = sxm; p.nseg = 1;
         p.W[0] = (const uint16_t*)W; p.swe = swe; p.ldw = nt ? swn : swk; p.nn = nn ? 1 : 0;
@@ -262,7 +262,7 @@ int moe_scatter2scatter(const void* X, int64_t sxm, int64_t sxk, const void* W, 
             if (A) {
                 // x A B = sum over 16-wide chunks c of x A[:, c] B[c, :]: a rank above 16 enters as several 16-wide K slabs
                 const int nh = (rank + 15) / 16;
-                void *At[MOE_MAX_SLABS] = {}, *LB[MOE_MAX_SLABS] = {}, *Q[MOE_MAX_SLABS] = {};
+                void *At[MOE_MAX_STRIDED_SLABS] = {}, *LB[MOE_MAX_STRIDED_SLABS] = {}, *Q[MOE_MAX_STRIDED_SLABS] = {};
                 for (int hf = 0; hf < nh; ++hf) {
                     At[hf] = ws.take(pack_bytes(E, K));
                     LB[hf] = ws.take(pack_bytes(E, N));
@@ -270,13 +270,17 @@ int moe_scatter2scatter(const void* X, int64_t sxm, int64_t sxk, const void* W, 
                     const int r0 = 16 * hf, rk = (rank - r0 < 16) ? rank - r0 : 16;
                     TRY(moe_launch_pack_lora((const uint16_t*)A + r0 * sar, sae, sak, sar, At[hf], E, K, rk, 1, S(stream)));
                     TRY(moe_launch_pack_lora((const uint16_t*)B + r0 * sbr, sbe, sbn, sbr, LB[hf], E, N, rk, 0, S(stream)));
-                    p.Q[hf] = (const uint16_t*)Q[hf]; p.LB[hf] = (const uint16_t*)LB[hf];
+                    if (hf < MOE_MAX_SLABS) { p.Q[hf] = (const uint16_t*)Q[hf]; p.LB[hf] = (const uint16_t*)LB[hf]; }
                 }
                 for (int hf = 0; hf < nh; hf += 2)   // two products over the same rows per launch
                     TRY(moe_launch_rows_lora2(X, hf + 1 < nh ? X : nullptr, sxm, At[hf], hf + 1 < nh ? At[hf + 1] : nullptr, Q[hf],
                                               hf + 1 < nh ? Q[hf + 1] : nullptr, nullptr, nullptr, 0, pos, pos64, offsets, off64, E, R, K,
                                               fan_out, x_grouped, scaling, nullptr, S(stream), nullptr, f16));
                 p.nslab = nh; p.slab_mode = 0;
+                if (nh > 1) {   // the chunks' buffers were taken in turn: a fixed stride from one chunk to the next
+                    p.q_slab_stride = (int64_t)((const uint16_t*)Q[1] - (const uint16_t*)Q[0]);
+                    p.lb_slab_stride = (int64_t)((const uint16_t*)LB[1] - (const uint16_t*)LB[0]);
+                }
             }
             return moe_launch_gemm_mfma(p, R, S(stream));
         }

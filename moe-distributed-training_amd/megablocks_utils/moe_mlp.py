@@ -341,11 +341,15 @@ class ScatterMoEBlock(nn.Module):
     """Drop-in for a Mixtral sparse-MoE block built the way the reference builds it: router weight (E, d), expert
     weights w1, w2, w3 stored (E*f, d) (megablocks_utils/sparse_mlp2.py:22-36, HF w2 transposed on load,
     shard_moe_utils.py:153-157), optional LoRA factors stored as peft_utils.py:37-38,68-70 does.  Returns
-    ``(hidden, None)`` like the patched ParallelMLP.forward (config_utils.py:75-92)."""
+    ``(hidden, None)`` like the patched ParallelMLP.forward (config_utils.py:75-92); with ``bias=True`` the block owns an
+    output bias (megablocks' ``ParallelMLP.bias``) and follows that method's bias branch (config_utils.py:80-84):
+    ``(hidden, bias)`` when ``return_bias`` is set, otherwise the single tensor ``hidden + bias``."""
 
     def __init__(self, hidden_size, ffn_hidden_size, num_experts, top_k=2, lora_r=0, lora_alpha=16.0,
-                 dtype=torch.bfloat16, device=None):
+                 dtype=torch.bfloat16, device=None, bias=False, return_bias=False):
         super().__init__()
+        self.return_bias = return_bias
+        self.bias = nn.Parameter(torch.zeros(hidden_size, dtype=dtype, device=device)) if bias else None
         self.hidden_size, self.ffn_hidden_size = hidden_size, ffn_hidden_size
         self.num_experts, self.top_k, self.lora_r, self.lora_alpha = num_experts, top_k, lora_r, lora_alpha
         kw = dict(dtype=dtype, device=device)
@@ -362,7 +366,7 @@ class ScatterMoEBlock(nn.Module):
                 nn.init.normal_(a, std=0.02)
                 self.register_parameter(f"lora_A_{n}", a)
                 self.register_parameter(f"lora_B_{n}", b)
-            for p in (self.router, self.w1, self.w2, self.w3):
+            for p in (self.router, self.w1, self.w2, self.w3) + (() if self.bias is None else (self.bias,)):
                 p.requires_grad_(False)
 
     def lora_views(self) -> Optional[LoraViews]:
@@ -375,10 +379,15 @@ class ScatterMoEBlock(nn.Module):
             v["a" + n[1]], v["b" + n[1]] = a, b
         return LoraViews(v["a1"], v["b1"], v["a3"], v["b3"], v["a2"], v["b2"])
 
-    def forward(self, hidden_states: torch.Tensor) -> Tuple[torch.Tensor, None]:
+    def forward(self, hidden_states: torch.Tensor):
         shape = hidden_states.shape
         x = hidden_states.reshape(-1, shape[-1])
         E, f, d = self.num_experts, self.ffn_hidden_size, self.hidden_size
         out, _, _ = moe_layer_forward(x, self.router, self.w1.view(E, f, d), self.w2.view(E, f, d),
                                       self.w3.view(E, f, d), self.top_k, self.lora_views(), self.lora_alpha)
-        return out.view(shape), None
+        out = out.view(shape)
+        if self.bias is not None:
+            if self.return_bias:
+                return out, self.bias
+            return out + self.bias
+        return out, None

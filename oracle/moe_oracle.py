@@ -17,9 +17,9 @@ Pins (tests/test_oracle_*.py): the index fixture and shapes of tests/test_scatte
 the docstring example of ops.py:45-49; transformers' MixtralSparseMoeBlock / MixtralTopKRouter as an
 independent library restatement of the block; torch.autograd.gradcheck in fp64; brute-force loops.
 The router's optional switches (``router_with_options``): bias, p-norm and jitter are pinned by the library
-routines they consist of (F.linear, torch.norm, a product).  Parity unpinned: the uniform expert assignment
-(megablocks' ``_uniform_expert_assignment`` is not part of the reference tree and no test of the reference uses it;
-restated from its name and its call site, config_utils.py:272-279).
+routines they consist of (F.linear, torch.norm, a product); the uniform expert assignment (megablocks'
+published ``_uniform_expert_assignment``, called at config_utils.py:272-279: experts 0..E-1 handed out in turn over the
+flattened assignments, ``arange % E``) by that closed form (tests/test_oracle_routing.py).
 """
 from __future__ import annotations
 

@@ -53,6 +53,8 @@ CASES = [
     (torch.bfloat16, 400, 4, 2, 256, 512, 32),   # rank above 16: the adapter enters as two 16-wide slabs
     (torch.bfloat16, 400, 4, 2, 256, 512, 64),   # four slabs in two MFMA steps
     (torch.bfloat16, 400, 4, 2, 256, 512, 40),   # three slabs, the last one partly filled
+    (torch.bfloat16, 400, 4, 2, 256, 512, 96),   # a rank above 64: six slabs at a fixed stride, two per step in a loop
+    (torch.float16, 400, 4, 2, 264, 256, 136),   # nine slabs (the last half empty), fp16, and a partial last K tile
     (torch.bfloat16, 1200, 96, 4, 256, 512, 16), # more than 64 experts (serial group lookup), top-4, every tile ragged
     (torch.bfloat16, 500, 4, 2, 64, 512, 16),    # a single K tile: the adapter slabs' LDS image is requested before the loop
     (torch.bfloat16, 500, 4, 2, 192, 300, 16),   # three K tiles: ... by the first trip through the loop
