@@ -304,7 +304,7 @@ def main():
         # fp32 runs on the generic (non matrix-core) kernels through the per-projection calls, which carry no stage timer: the
         # whole step stands for the kernel, against the fp32 vector peak
         peak = 157.3
-        roofline = {"bound": "mfma", "kernel": "generic_gemm_kernel (whole step: a few microseconds of work, launch bound)",
+        roofline = {"bound": "valu", "kernel": "generic_gemm_kernel (whole step: a few microseconds of fp32 vector arithmetic, launch bound)",
                     "achieved": round(tflops, 4), "peak": peak, "unit": "TFLOP/s", "frac": round(tflops / peak, 6), "traffic": None}
     what = ("fwd+bwd" if cfg["bwd"] else "fwd")
     metric = "MoE-layer fwd+bwd TFLOP/s & % bf16 MFMA peak, Mixtral shape T=4096, 1 GPU" if args.workload == "mixtral_fwd_bwd_lora" \
