@@ -181,24 +181,27 @@ def test_scatter2scatter_out_argument_and_empty(dev, oracle):
     ([130, 5, 0, 260], 264, 136),            # K and N not multiples of the 256 tile: edge columns are masked
     ([1000, 3000], 768, 2304),               # several panels of n tiles, long contraction
 ])
-def test_group_bwd_w_matrix_cores(dev, oracle, counts, K, N):
-    """bf16 DW[e] = X_e^T DY_e (scattermoe group_bwd_W, full fine-tuning) against the fp32 per-expert matmul; rows of
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_group_bwd_w_matrix_cores(dev, oracle, counts, K, N, dtype):
+    """bf16 / fp16 DW[e] = X_e^T DY_e (scattermoe group_bwd_W, full fine-tuning) against the fp32 per-expert matmul; rows of
     the next group must not leak into a group's last, partial contraction step, an empty group gives zeros."""
     ops = _ops()
     torch.manual_seed(11)
     E = len(counts)
     eo = torch.tensor(counts).cumsum(0)
     R = int(eo[-1])
-    X = torch.randn(R, K).bfloat16(); DY = torch.randn(R, N).bfloat16()
+    X = torch.randn(R, K).to(dtype); DY = (torch.randn(R, N) * 0.25).to(dtype)
     ref = oracle.group_bwd_W(DY, X, eo, E)
     for offs in (eo.to(dev), eo.int().to(dev)):
         dW = ops.group_bwd_W(DY.to(dev), X.to(dev), offs, E)
-        assert dW.shape == (E, K, N) and dW.dtype == torch.bfloat16
+        assert dW.shape == (E, K, N) and dW.dtype == dtype
         for e in range(E):
             if counts[e] == 0:
                 assert float(dW[e].abs().max()) == 0.0
             else:
-                assert rel(dW[e], ref[e]) < TOL[torch.bfloat16]
+                assert rel(dW[e], ref[e]) < TOL[dtype]
+    if dtype != torch.bfloat16:
+        return
     # row-strided operands (column slices of wider buffers) take the same kernel
     Xw = torch.randn(R, K + 64).bfloat16().to(dev); DYw = torch.randn(R, N + 8).bfloat16().to(dev)
     dW = ops.group_bwd_W(DYw[:, 8:], Xw[:, 64:], eo.to(dev), E)
@@ -227,7 +230,7 @@ def test_group_bwd_w_mixtral_shape(dev, oracle):
 
 @pytest.mark.parametrize("dtype,K,N,r", [(torch.float32, 150, 140, 4), (torch.bfloat16, 256, 512, 16), (torch.bfloat16, 256, 512, 64),
                                          (torch.bfloat16, 4096, 1024, 16), (torch.bfloat16, 96, 160, 8),
-                                         (torch.float16, 130, 70, 16)])
+                                         (torch.float16, 130, 70, 16), (torch.float16, 256, 512, 16), (torch.float16, 512, 288, 48)])
 def test_group_bwd_ab_full_reduction(dev, oracle, dtype, K, N, r):
     """K and N above 128 on purpose: every N tile must contribute to dA and every K tile to dB."""
     ops = _ops()
@@ -311,7 +314,7 @@ def _run_parallel_linear(dev, oracle, dtype, T, E, k, K, N, r, gates, gin, gout,
 
 
 @pytest.mark.parametrize("dtype,K,N,r", [(torch.float32, 128, 16, 16), (torch.bfloat16, 256, 384, 16), (torch.bfloat16, 200, 136, 16),
-                                         (torch.bfloat16, 256, 384, 32)])
+                                         (torch.bfloat16, 256, 384, 32), (torch.float16, 256, 384, 16)])
 @pytest.mark.parametrize("gates,gin,gout", [(False, False, True), (False, True, False), (True, False, False), (False, False, False), (False, True, True)])
 def test_parallel_linear_lora_autograd(dev, oracle, dtype, K, N, r, gates, gin, gout):
     _run_parallel_linear(dev, oracle, dtype, 333, 4, 2, K, N, r, gates, gin, gout)
