@@ -49,6 +49,8 @@ WORKLOADS = {
                                  desc="Mixtral-8x7B MoE layer fwd+bwd, T=4096, bf16, top-2, LoRA r=16 alpha=32 (BASELINE configs[2])"),
     "mixtral_fwd_bwd_lora_r32": dict(T=4096, d=4096, f=14336, E=8, k=2, r=32, bwd=True, skew=False,
                                      desc="Mixtral-8x7B MoE layer fwd+bwd, T=4096, bf16, top-2, LoRA r=32 alpha=32 (adapters as two 16-wide rank chunks)"),
+    "mixtral_fwd_bwd_lora_fp16": dict(T=4096, d=4096, f=14336, E=8, k=2, r=16, bwd=True, skew=False, dtype="fp16",
+                                      desc="Mixtral-8x7B MoE layer fwd+bwd, T=4096, fp16 (the reference's fp16 switch), top-2, LoRA r=16 alpha=32"),
     "mixtral_fwd": dict(T=4096, d=4096, f=14336, E=8, k=2, r=0, bwd=False, skew=False,
                         desc="Mixtral-8x7B MoE layer forward, T=4096, bf16, top-2 (BASELINE configs[1])"),
     "mixtral_fwd_bwd_full": dict(T=4096, d=4096, f=14336, E=8, k=2, r=0, bwd=True, skew=False, train_base=True,
@@ -82,7 +84,7 @@ def make_inputs(cfg, dev, seed=0):
     import torch
     g = torch.Generator(device=dev).manual_seed(seed)
     T, d, f, E, r = cfg["T"], cfg["d"], cfg["f"], cfg["E"], cfg["r"]
-    bf = torch.float32 if cfg.get("dtype") == "fp32" else torch.bfloat16
+    bf = {"fp32": torch.float32, "fp16": torch.float16}.get(cfg.get("dtype"), torch.bfloat16)
 
     def rn(*shape, std=1.0):
         return (torch.randn(*shape, generator=g, device=dev, dtype=torch.float32) * std).to(bf)
@@ -290,6 +292,7 @@ def main():
                   "bwd.group_bwd_w": 2 * R * cfg["d"] * cfg["f"]}
     gemm_stages = {k_: v for k_, v in stages.items() if k_ in gemm_flops}
     fp32 = cfg.get("dtype") == "fp32"
+    fp16 = cfg.get("dtype") == "fp16"   # same dense MFMA peak as bf16 (2.5 PFLOP/s)
     if gemm_stages:
         dom = max(gemm_stages, key=gemm_stages.get)
         ach = gemm_flops[dom] / (gemm_stages[dom] * 1e-3) / 1e12
@@ -308,12 +311,12 @@ def main():
                     "achieved": round(tflops, 4), "peak": peak, "unit": "TFLOP/s", "frac": round(tflops / peak, 6), "traffic": None}
     what = ("fwd+bwd" if cfg["bwd"] else "fwd")
     metric = "MoE-layer fwd+bwd TFLOP/s & % bf16 MFMA peak, Mixtral shape T=4096, 1 GPU" if args.workload == "mixtral_fwd_bwd_lora" \
-        else f"MoE-layer {what} TFLOP/s & % {'fp32' if fp32 else 'bf16 MFMA'} peak, workload {args.workload}, 1 GPU"
+        else f"MoE-layer {what} TFLOP/s & % {'fp32' if fp32 else 'fp16 MFMA' if fp16 else 'bf16 MFMA'} peak, workload {args.workload}, 1 GPU"
     result = {
         "metric": metric,
         "value": round(tflops, 4 if fp32 else 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(dt * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "fp32" if fp32 else "bf16", "data": "synthetic",
+        "dtype": "fp32" if fp32 else "fp16" if fp16 else "bf16", "data": "synthetic",
         "config": {"workload": cfg["desc"], "tokens": cfg["T"], "d_model": cfg["d"], "d_ff": cfg["f"],
                    "experts": cfg["E"], "top_k": cfg["k"], "lora_rank": cfg["r"]},
         "tokens_per_s": round(cfg["T"] / dt, 1),
