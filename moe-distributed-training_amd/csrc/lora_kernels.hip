@@ -10,6 +10,21 @@
 
 namespace {
 
+// Two jobs of a launch that read the same rows (x A1 and x A3, say) should run side by side on one XCD, so that the rows
+// the first fetches serve the second from that XCD's L2: workgroups are dispatched to the 8 XCDs in turn by their linear
+// number, so a one-dimensional grid deals units out in groups of 8 -- unit 8g + i of job j is workgroup (g * jobs + j) * 8 + i,
+// eight workgroups behind its twin of the other job and on the same XCD.
+constexpr int JOB_GROUP = 8;
+__device__ __forceinline__ void unit_and_job(int njobs, int64_t* unit, int* job)
+{
+    const int64_t id = blockIdx.x;
+    const int64_t group = id / (JOB_GROUP * njobs);
+    const int within = (int)(id % (JOB_GROUP * njobs));
+    *job = within / JOB_GROUP;
+    *unit = group * JOB_GROUP + within % JOB_GROUP;
+}
+inline unsigned job_grid(int64_t units, int njobs) { return (unsigned)((units + JOB_GROUP - 1) / JOB_GROUP * JOB_GROUP * njobs); }
+
 // (fragment order covers K rounded up to whole 32-wide fragments; positions at or past K hold zeros, so a consumer may
 // feed them anything finite)
 __global__ void pack_lora_kernel(const uint16_t* __restrict__ src, int64_t se, int64_t sk, int64_t sr,
@@ -90,7 +105,7 @@ static_assert(RL_KSTEPS == RL_WAVES, "one K step per wave and stage");
 // values per lane) are then read from LDS.  Loading the fragments straight from global memory would make adjacent
 // lanes touch different rows, which the memory pipeline handles one lane at a time.  All global loads of the loop are
 // inline assembly with explicit s_waitcnt: compiler-managed loads would wait for the prefetches queued behind them.
-// one or two jobs per launch (blockIdx.y): same rows, shapes and scaling, different operand / output pointers
+// one or two jobs per launch (see unit_and_job): same rows, shapes and scaling, different operand / output pointers
 struct RowsLoraJob { const uint16_t* X; const uint16_t* Af; uint16_t* Q; uint16_t* Qt; uint16_t* Qs; };   // Qs: optional row-major copy scaled like Qt
 // ROWS = 32 rows per workgroup, or 16 when a launch of 32-row tiles would leave most compute units with a single
 // workgroup (and so with too few loads in flight)
@@ -99,16 +114,19 @@ __global__ void __launch_bounds__(RL_THREADS) rows_lora_kernel(const RowsLoraJob
                                                                int64_t ldqt, const void* __restrict__ pos, int pos64,
                                                                const void* __restrict__ offsets, int off64, int E,
                                                                int64_t K, int fan_out, int x_grouped, float scaling,
-                                                               const float* __restrict__ qt_row_scale)
+                                                               const float* __restrict__ qt_row_scale, int njobs)
 {
-    const RowsLoraJob& job = blockIdx.y ? job1 : job0;
+    int64_t tile_id;
+    int job_id;
+    unit_and_job(njobs, &tile_id, &job_id);
+    const RowsLoraJob& job = job_id ? job1 : job0;
     const uint16_t* __restrict__ X = job.X;
     const uint16_t* __restrict__ Af = job.Af;
     uint16_t* __restrict__ Q = job.Q;
     uint16_t* __restrict__ Qt = job.Qt;
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
     RowTile rt;
-    if (!find_row_tile(offsets, off64, E, ROWS, blockIdx.x, &rt)) return;
+    if (!find_row_tile(offsets, off64, E, ROWS, tile_id, &rt)) return;
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int i = lane & 15, g = lane >> 4;
     const int expert = __builtin_amdgcn_readfirstlane(rt.expert);
@@ -207,7 +225,7 @@ constexpr int XTP_COLS = 4 * XTP_WCOLS;  // columns per workgroup
 // (8 x 16-byte loads) and transposes them in registers into 8 column fragments; the P fragment is one 16-byte
 // load from the transposed copy Pt.  Each wave owns 128 columns and walks the tile's rows 32 at a time with the
 // next block's loads in flight, so there is no cross-wave reduction.
-// one or two jobs per launch (blockIdx.z): same rows and shapes, different operands / outputs; job j's partials start
+// one or two jobs per launch (see unit_and_job): same rows and shapes, different operands / outputs; job j's partials start
 // at partial + j * partial_stride
 struct XtpJob { const uint16_t* X; const uint16_t* Pt; uint16_t* out; int64_t soe, sok, sor; int rank; };   // rank: columns written (<= 16)
 template <typename Num>
@@ -217,17 +235,23 @@ __global__ void __launch_bounds__(XTP_THREADS) xtp_partial_kernel(const XtpJob j
                                                                   const float* __restrict__ p_row_scale,
                                                                   float* __restrict__ partial, int64_t partial_stride,
                                                                   const void* __restrict__ offsets, int off64, int E,
-                                                                  int64_t R, int64_t K)
+                                                                  int64_t R, int64_t K, int njobs)
 {
-    const XtpJob& job = blockIdx.z ? job1 : job0;
+    // unit = (row tile, column block), column block fastest
+    int64_t unit;
+    int job_id;
+    unit_and_job(njobs, &unit, &job_id);
+    const int64_t kblocks = (K + XTP_COLS - 1) / XTP_COLS;
+    const int64_t tile_id = unit / kblocks, kblock = unit % kblocks;
+    const XtpJob& job = job_id ? job1 : job0;
     const uint16_t* __restrict__ X = job.X;
     const uint16_t* __restrict__ Pt = job.Pt;
-    partial += (int64_t)blockIdx.z * partial_stride;
+    partial += (int64_t)job_id * partial_stride;
     RowTile rt;
-    if (!find_row_tile(offsets, off64, E, XTP_RC, blockIdx.y, &rt)) return;
+    if (!find_row_tile(offsets, off64, E, XTP_RC, tile_id, &rt)) return;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int i = lane & 15, g = lane >> 4;
-    const int64_t kcol = (int64_t)blockIdx.x * XTP_COLS + wave * XTP_WCOLS + 8 * i;
+    const int64_t kcol = kblock * XTP_COLS + wave * XTP_WCOLS + 8 * i;
     const bool col_ok = kcol < K;  // K % 8 == 0: a lane's 8 columns are all in or all out
     f32x4_t acc[8];
 #pragma unroll
@@ -289,13 +313,13 @@ __global__ void __launch_bounds__(XTP_THREADS) xtp_partial_kernel(const XtpJob j
         }
     }
     // acc[j][reg]: X column kcol0 + 8*(g*4 + reg) + j (MFMA row g*4+reg), P column i
-    float* out = partial + ((int64_t)blockIdx.y * K + (int64_t)blockIdx.x * XTP_COLS + wave * XTP_WCOLS) * 16;
+    float* out = partial + (tile_id * K + kblock * XTP_COLS + wave * XTP_WCOLS) * 16;
 #pragma unroll
     for (int j = 0; j < 8; ++j)
 #pragma unroll
         for (int reg = 0; reg < 4; ++reg) {
             const int c = 8 * (g * 4 + reg) + j;
-            if ((int64_t)blockIdx.x * XTP_COLS + wave * XTP_WCOLS + c < K) out[c * 16 + i] = acc[j][reg];
+            if (kblock * XTP_COLS + wave * XTP_WCOLS + c < K) out[c * 16 + i] = acc[j][reg];
         }
 }
 
@@ -452,11 +476,11 @@ int moe_launch_rows_lora2(const void* X, const void* X2, int64_t ldx, const void
     const int cus = moe_device_cus();
     const int64_t tiles32 = (R / 32 + E) * (two ? 2 : 1);
     if (tiles32 >= 3 * (int64_t)cus / 2) {
-        hipLaunchKernelGGL((f16 ? rows_lora_kernel<32, NumF16> : rows_lora_kernel<32, NumBf16>), dim3((unsigned)(R / 32 + E), two ? 2u : 1u), dim3(RL_THREADS), rl_lds(32), stream, j0, j1,
-                           ldx, ldqt, pos, pos64, offsets, off64, E, K, fan_out, x_grouped, scaling, qt_row_scale);
+        hipLaunchKernelGGL((f16 ? rows_lora_kernel<32, NumF16> : rows_lora_kernel<32, NumBf16>), dim3(job_grid(R / 32 + E, two ? 2 : 1)), dim3(RL_THREADS), rl_lds(32), stream, j0, j1,
+                           ldx, ldqt, pos, pos64, offsets, off64, E, K, fan_out, x_grouped, scaling, qt_row_scale, two ? 2 : 1);
     } else {
-        hipLaunchKernelGGL((f16 ? rows_lora_kernel<16, NumF16> : rows_lora_kernel<16, NumBf16>), dim3((unsigned)(R / 16 + E), two ? 2u : 1u), dim3(RL_THREADS), rl_lds(16), stream, j0, j1,
-                           ldx, ldqt, pos, pos64, offsets, off64, E, K, fan_out, x_grouped, scaling, qt_row_scale);
+        hipLaunchKernelGGL((f16 ? rows_lora_kernel<16, NumF16> : rows_lora_kernel<16, NumBf16>), dim3(job_grid(R / 16 + E, two ? 2 : 1)), dim3(RL_THREADS), rl_lds(16), stream, j0, j1,
+                           ldx, ldqt, pos, pos64, offsets, off64, E, K, fan_out, x_grouped, scaling, qt_row_scale, two ? 2 : 1);
     }
     return moe_launch_status();
 }
@@ -492,9 +516,10 @@ int moe_launch_xtp2(const void* X, const void* X2, int64_t ldx, const void* pos,
     const XtpJob j1 = two ? XtpJob{(const uint16_t*)X2, (const uint16_t*)Pt2, (uint16_t*)out2, so2[0], so2[1], so2[2], rank2} : j0;
     const int64_t pstride = (int64_t)(one / sizeof(float));
     if (R > 0) {
-        dim3 grid((unsigned)((K + XTP_COLS - 1) / XTP_COLS), (unsigned)tiles, two ? 2u : 1u);
-        hipLaunchKernelGGL(f16 ? xtp_partial_kernel<NumF16> : xtp_partial_kernel<NumBf16>, grid, dim3(XTP_THREADS), 0, stream, j0, j1, ldx, pos, pos64, fan_out, ldpt,
-                           p_row_scale, (float*)workspace, pstride, offsets, off64, E, R, K);
+        const int64_t units = ((K + XTP_COLS - 1) / XTP_COLS) * tiles;
+        if (units * 2 + 16 >= ((int64_t)1 << 31)) return MOE_ERR_UNSUPPORTED;
+        hipLaunchKernelGGL(f16 ? xtp_partial_kernel<NumF16> : xtp_partial_kernel<NumBf16>, dim3(job_grid(units, two ? 2 : 1)), dim3(XTP_THREADS), 0, stream, j0, j1, ldx, pos, pos64, fan_out, ldpt,
+                           p_row_scale, (float*)workspace, pstride, offsets, off64, E, R, K, two ? 2 : 1);
     }
     dim3 rgrid((unsigned)((K * 4 + 255) / 256), (unsigned)E, two ? 2u : 1u);
     hipLaunchKernelGGL(f16 ? xtp_reduce_kernel<NumF16> : xtp_reduce_kernel<NumBf16>, rgrid, dim3(256), 0, stream, (const float*)workspace, pstride, j0, j1, offsets,
