@@ -709,10 +709,12 @@ int moe_mlp_bwd(const void* dy, int64_t lddy, int dy_grouped, int dy_fan_out, co
         if (fuse_rc) {   // the products over each column tile came out of the dh GEMM's epilogue: add the tiles, scale, round
             const size_t cone = cc_bytes(R, f) / 2 / sizeof(float);
             TRY(moe_launch_cc_reduce2(ccw, ccw + cone, (int)((f + 255) / 256), R, scaling, pqp(1, 0), pqp(2, 0), pqp(4, 0), pqp(5, 0), ldt, st, f16));
-        } else
-        for (int c = 0; c < C; ++c)
-            TRY(moe_launch_rows_lora2(dgate, dup, f, bt1[c], bt3[c], pqp(1, c), pqp(2, c), pqp(4, c), pqp(5, c), ldt, nullptr, 0, offsets,
+        } else {   // two chunks: the chunks of one adapter share a launch, so that dgate and dup are each read once
+            TRY(moe_launch_rows_lora2(dgate, dgate, f, bt1[0], bt1[1], pqp(1, 0), pqp(1, 1), pqp(4, 0), pqp(4, 1), ldt, nullptr, 0, offsets,
                                       off64, E, R, f, 1, 1, scaling, nullptr, st, nullptr, f16));
+            TRY(moe_launch_rows_lora2(dup, dup, f, bt3[0], bt3[1], pqp(2, 0), pqp(2, 1), pqp(5, 0), pqp(5, 1), ldt, nullptr, 0, offsets,
+                                      off64, E, R, f, 1, 1, scaling, nullptr, st, nullptr, f16));
+        }
     }
     {
         MoeGemmParams p = {};
@@ -743,9 +745,12 @@ int moe_mlp_bwd(const void* dy, int64_t lddy, int dy_grouped, int dy_fan_out, co
             const int rk = (rank - 16 * c < 16) ? rank - 16 * c : 16;
             TRY(moe_launch_xtp2(x, x, ldx, pos, pos64, fan_out, pqp(4, c), pqp(5, c), ldt, nullptr, (uint16_t*)lg[0] + 16 * c * gs[2],
                                 (uint16_t*)lg[2] + 16 * c * gs[8], sa1, sa3, rk, rk, offsets, off64, E, R, d, 1.f, xw, xb, st, f16));
-            if (!fuse_rc)
-            TRY(moe_launch_xtp2(dgate, dup, f, nullptr, 0, 1, svp(3, c), svp(4, c), ldt, nullptr, (uint16_t*)lg[1] + 16 * c * gs[4],
-                                (uint16_t*)lg[3] + 16 * c * gs[10], sb1, sb3, rk, rk, offsets, off64, E, R, f, 1.f, xw, xb, st, f16));
+        }
+        if (!fuse_rc) {   // two chunks: the chunks of one adapter share a launch, so that dgate and dup are each read once
+            TRY(moe_launch_xtp2(dgate, dgate, f, nullptr, 0, 1, svp(3, 0), svp(3, 1), ldt, nullptr, lg[1], (uint16_t*)lg[1] + 16 * gs[4],
+                                sb1, sb1, 16, rank - 16, offsets, off64, E, R, f, 1.f, xw, xb, st, f16));
+            TRY(moe_launch_xtp2(dup, dup, f, nullptr, 0, 1, svp(4, 0), svp(4, 1), ldt, nullptr, lg[3], (uint16_t*)lg[3] + 16 * gs[10],
+                                sb3, sb3, 16, rank - 16, offsets, off64, E, R, f, 1.f, xw, xb, st, f16));
         }
     }
     return MOE_OK;
