@@ -49,6 +49,8 @@ WORKLOADS = {
                                  desc="Mixtral-8x7B MoE layer fwd+bwd, T=4096, bf16, top-2, LoRA r=16 alpha=32 (BASELINE configs[2])"),
     "mixtral_fwd_bwd_lora_r32": dict(T=4096, d=4096, f=14336, E=8, k=2, r=32, bwd=True, skew=False,
                                      desc="Mixtral-8x7B MoE layer fwd+bwd, T=4096, bf16, top-2, LoRA r=32 alpha=32 (adapters as two 16-wide rank chunks)"),
+    "mixtral_fwd_bwd_lora_r64": dict(T=4096, d=4096, f=14336, E=8, k=2, r=64, bwd=True, skew=False,
+                                     desc="Mixtral-8x7B MoE layer fwd+bwd, T=4096, bf16, top-2, LoRA r=64 alpha=32 (adapters as four 16-wide rank chunks)"),
     "mixtral_fwd_bwd_lora_fp16": dict(T=4096, d=4096, f=14336, E=8, k=2, r=16, bwd=True, skew=False, dtype="fp16",
                                       desc="Mixtral-8x7B MoE layer fwd+bwd, T=4096, fp16 (the reference's fp16 switch), top-2, LoRA r=16 alpha=32"),
     "mixtral_fwd": dict(T=4096, d=4096, f=14336, E=8, k=2, r=0, bwd=False, skew=False,

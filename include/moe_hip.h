@@ -190,8 +190,9 @@ int moe_swiglu_bwd(const void* gate, const void* up, const void* dh, void* dgate
  * Forward:  gate = x W1^T (+lora), up = x W3^T (+lora)   [one dual-weight GEMM, x gathered by pos/fan_out]
  *           h = silu(gate) * up                          [fused epilogue; gate/up saved when save_gate_up]
  *           y[out_row] = h W2 (+lora)                    [out_row = y_grouped ? m : pos[m]]
- * `saved` receives the low-rank interims needed by the backward (moe_mlp_saved_bytes).  Adapter rank <= 32 (an adapter is
- * worked through as one or two chunks of 16 rank columns); higher ranks: use the per-projection entry points. */
+ * `saved` receives the low-rank interims needed by the backward (moe_mlp_saved_bytes).  Adapter rank <= 128 (an adapter is
+ * worked through as up to eight chunks of 16 rank columns; one chunk has its products with h, dgate and dup folded into
+ * the GEMM epilogues, more chunks take separate passes over those tensors); higher ranks: use the per-projection entry points. */
 size_t moe_mlp_workspace_bytes(int64_t R, int E, int64_t d, int64_t f, int rank);
 size_t moe_mlp_saved_bytes(int64_t R, int rank);
 int moe_mlp_fwd(const void* x, int64_t ldx, const void* w1, const void* w3, const void* w2, const void* const* lora,

@@ -656,43 +656,49 @@ __global__ void __launch_bounds__(NTHREADS) grouped_gemm_mfma_kernel(const MoeGe
     // are read from the LDS image that the main loop fetched as "the tile after the last" (the gate/up launch 1.5 %
     // faster than with the round trip to memory here); three or four come straight from global memory, all fragments
     // requested before the first of them is used, so that the tile pays one memory round trip, not one per fragment.
-    // More than MOE_MAX_SLABS slabs (an adapter rank above 64; general variant, every slab feeds every column): the slabs
+    // More than MOE_MAX_SLABS slabs (an adapter rank above 64, above 32 for the gate/up pair; general variant): the slabs
     // are slab_stride-spaced copies of Q[0] / LB[0] and are worked through two per MFMA step in a loop, each step's
     // fragments straight from global memory -- one round trip per 32 rank columns, paid only by such ranks.
     if constexpr (KTAIL) {
         if (p.nslab > MOE_MAX_SLABS) {
             const int kc = (lane >> 4) & 1;
             const bool upper = lane >= 32;
+            const int ngroups = p.slab_mode == 0 ? 1 : 2;   // slab_mode 1: gate slabs, then up slabs
+            const int per_group = p.nslab / ngroups;
 #pragma unroll 1
-            for (int lo = 0; lo < p.nslab; lo += 2) {
-                const bool has_hi = lo + 1 < p.nslab;
-                const int src = (upper && has_hi) ? lo + 1 : lo;
-                const bool live = !upper || has_hi;
-                const uint16_t* Q = p.Q[0] + (int64_t)src * p.q_slab_stride;
-                const uint16_t* LB = p.LB[0] + (int64_t)src * p.lb_slab_stride + (int64_t)expert * p.N * 16;
-                bf16x8_t ta[MB], tb[NB];
+            for (int grp = 0; grp < ngroups; ++grp) {
+#pragma unroll 1
+                for (int l = 0; l < per_group; l += 2) {
+                    const bool has_hi = l + 1 < per_group;
+                    const int src = grp * per_group + ((upper && has_hi) ? l + 1 : l);
+                    const bool live = !upper || has_hi;
+                    const uint16_t* Q = p.Q[0] + (int64_t)src * p.q_slab_stride;
+                    const uint16_t* LB = p.LB[0] + (int64_t)src * p.lb_slab_stride + (int64_t)expert * p.N * 16;
+                    bf16x8_t ta[MB], tb[NB];
 #pragma unroll
-                for (int nb = 0; nb < NB; ++nb) {
-                    int64_t n = n0 + wn * WTN + nb * 16 + (lane & 15);
-                    if (n >= p.N) n = p.N - 1;
-                    bf16x8_t v = {};
-                    if (live) v = *(const bf16x8_t*)(LB + n * 16 + 8 * kc);
-                    tb[nb] = v;
-                }
-#pragma unroll
-                for (int mb = 0; mb < MB; ++mb) {
-                    int r = wm * WTM + mb * 16 + (lane & 15);
-                    if (r >= nrows) r = nrows - 1;
-                    bf16x8_t v = {};
-                    if (live) v = *(const bf16x8_t*)(Q + (row0 + r) * 16 + 8 * kc);
-                    ta[mb] = v;
-                }
-#pragma unroll
-                for (int mb = 0; mb < MB; ++mb)
-                    if (mb < mb_cnt) {
-#pragma unroll
-                        for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = Num::mfma(tb[nb], ta[mb], acc[mb][nb]);
+                    for (int nb = 0; nb < NB; ++nb) {
+                        int64_t n = (EPI_IS_PAIR(EPI)) ? n0 + wn * (WTN / 2) + (nb % NBH) * 16 + (lane & 15) : n0 + wn * WTN + nb * 16 + (lane & 15);
+                        if (n >= p.N) n = p.N - 1;
+                        bf16x8_t v = {};
+                        if (live) v = *(const bf16x8_t*)(LB + n * 16 + 8 * kc);
+                        tb[nb] = v;
                     }
+#pragma unroll
+                    for (int mb = 0; mb < MB; ++mb) {
+                        int r = wm * WTM + mb * 16 + (lane & 15);
+                        if (r >= nrows) r = nrows - 1;
+                        bf16x8_t v = {};
+                        if (live) v = *(const bf16x8_t*)(Q + (row0 + r) * 16 + 8 * kc);
+                        ta[mb] = v;
+                    }
+#pragma unroll
+                    for (int mb = 0; mb < MB; ++mb)
+                        if (mb < mb_cnt) {
+#pragma unroll
+                            for (int nb = 0; nb < NB; ++nb)
+                                if (p.slab_mode == 0 || nb / NBH == grp) acc[mb][nb] = Num::mfma(tb[nb], ta[mb], acc[mb][nb]);
+                        }
+                }
             }
         }
     }
@@ -1218,8 +1224,8 @@ template <bool NN, int EPI, typename Num, bool KTAIL> int launch_typed(const Moe
 // the kernel variant for the launch's 16-bit storage type
 template <bool NN, int EPI> int launch_variant(const MoeGemmParams& p, int64_t R, hipStream_t stream)
 {
-    if (p.K % BK != 0 || p.nslab > MOE_MAX_SLABS) {   // a partial last K tile, a rank above 64: the plain epilogue only (the fused layer's shapes are whole tiles, its ranks smaller)
-        if constexpr (EPI == MOE_EPI_STORE)
+    if (p.K % BK != 0 || p.nslab > MOE_MAX_SLABS) {   // a partial last K tile, many slabs: the plain epilogue, and the two SwiGLU epilogues without fused adapter products
+        if constexpr (EPI == MOE_EPI_STORE || (!NN && (EPI == MOE_EPI_SWIGLU || EPI == MOE_EPI_SWIGLU_BWD)))
             return p.f16 ? launch_typed<NN, EPI, NumF16, true>(p, R, stream) : launch_typed<NN, EPI, NumBf16, true>(p, R, stream);
         else
             return MOE_ERR_UNSUPPORTED;
@@ -1272,7 +1278,11 @@ bool moe_gemm_mfma_supported(const MoeGemmParams& p, int64_t R)
     for (int i = 0; i < MOE_MAX_SLABS; ++i)
         if (!al16(p.Q[i]) || !al16(p.LB[i])) return false;   // (slabs beyond these: multiples of 16 bytes from Q[0] / LB[0], checked below)
     if (p.nseg < 1 || p.nseg > 2 || p.nslab < 0 || (p.slab_mode == 1 && p.nslab % 2 != 0)) return false;
-    if (p.nslab > MOE_MAX_SLABS && (p.epi != MOE_EPI_STORE || p.slab_mode != 0 || p.nslab > MOE_MAX_STRIDED_SLABS || p.q_slab_stride % 8 != 0 || p.lb_slab_stride % 8 != 0)) return false;
+    if (p.K % BK != 0 && p.epi != MOE_EPI_STORE) return false;   // a partial last K tile: the plain epilogue only
+    if (p.nslab > MOE_MAX_SLABS) {
+        const bool epi_ok = p.epi == MOE_EPI_STORE || (!p.nn && (p.epi == MOE_EPI_SWIGLU || p.epi == MOE_EPI_SWIGLU_BWD));
+        if (!epi_ok || (p.slab_mode == 1) != (p.epi == MOE_EPI_SWIGLU) || p.nslab > MOE_MAX_STRIDED_SLABS || p.q_slab_stride % 8 != 0 || p.lb_slab_stride % 8 != 0) return false;
+    }
     // 32-bit byte offsets: gathered A rows from the start of X (grouped ones from the tile's first row), weights from
     // the start of one expert's matrix, grouped outputs and the saved gate / up from the tile's first row; scattered
     // output rows from the start of Y while Y spans less than 2 GiB, 64-bit addresses beyond (y_wide, set at launch)

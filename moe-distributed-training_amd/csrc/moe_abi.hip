@@ -449,10 +449,13 @@ size_t moe_mlp_workspace_bytes(int64_t R, int E, int64_t d, int64_t f, int rank)
 
 size_t moe_mlp_saved_bytes(int64_t R, int rank) { return rank > 0 ? (size_t)((rank + 15) / 16) * 6 * q_bytes(R) : 256; }
 
+// An adapter of rank r enters the fused layer as C = ceil(r / 16) chunks of 16 rank columns; the gate/up launch takes
+// the chunks of both its adapters as K slabs, which bounds C
+constexpr int MLP_MAX_CHUNKS = MOE_MAX_STRIDED_SLABS / 2;
 static bool mlp_shapes_ok(int64_t d, int64_t f, int64_t ldx, int rank, const void* a, const void* b, const void* c,
                           const void* x)
 {
-    return d % 64 == 0 && f % 64 == 0 && ldx % 8 == 0 && rank <= 32 && aligned16(a) && aligned16(b) && aligned16(c) &&
+    return d % 64 == 0 && f % 64 == 0 && ldx % 8 == 0 && rank <= 16 * MLP_MAX_CHUNKS && aligned16(a) && aligned16(b) && aligned16(c) &&
            aligned16(x);
 }
 // What the grouped GEMM's 32-bit offsets allow, checked before anything is enqueued: gathered rows are addressed from
@@ -486,38 +489,56 @@ int moe_mlp_fwd(const void* x, int64_t ldx, const void* w1, const void* w3, cons
     void* skws = ws.take(sk_bytes_mlp(R, E, d, f));
     bool counters_clean = has_lora;   // K-split counters: zeroed by the adapter pack launch; a GEMM launch that uses them leaves them zero
     // An adapter of rank r is worked through as C = ceil(r / 16) independent 16-wide chunks of its rank columns:
-    // x A B = sum_c (x A[:, c]) B[c, :].  saved: per chunk c, Q1, Q3, Q2, Qt1, Qt3, Qt2 (six q_bytes blocks).
+    // x A B = sum_c (x A[:, c]) B[c, :].  saved: six groups of C q_bytes blocks (one per chunk): Q1, Q3, Q2, Qt1, Qt3, Qt2.
+    // The chunks of a group lie at one stride, and so do the packed B-side images, so that a launch with many slabs
+    // finds slab s at base + s * stride (the gate/up launch: Q1 chunks then Q3 chunks, lb1 chunks then lb3 chunks).
     const int C = has_lora ? (rank + 15) / 16 : 0;
-    auto svp = [&](int which, int c) { return sv + ((size_t)c * 6 + which) * qb; };   // which: 0 Q1, 1 Q3, 2 Q2, 3 Qt1, 4 Qt3, 5 Qt2
-    void *At1[2] = {}, *At3[2] = {}, *lb1[2] = {}, *lb3[2] = {}, *At2c[2] = {}, *lb2[2] = {};
+    auto svp = [&](int which, int c) { return sv + ((size_t)which * C + c) * qb; };   // which: 0 Q1, 1 Q3, 2 Q2, 3 Qt1, 4 Qt3, 5 Qt2
+    const size_t pbd = pack_bytes(E, d), pbf = pack_bytes(E, f);
+    void *At1[MLP_MAX_CHUNKS] = {}, *At3[MLP_MAX_CHUNKS] = {}, *At2c[MLP_MAX_CHUNKS] = {};
+    uint8_t *lb13 = nullptr, *lb2 = nullptr;
+    auto lb1 = [&](int c) { return lb13 + (size_t)c * pbf; };
+    auto lb3 = [&](int c) { return lb13 + (size_t)(C + c) * pbf; };
+    auto lb2c = [&](int c) { return lb2 + (size_t)c * pbd; };
+    // the slabs of a launch: by their own pointers while they fit, else by base and stride
+    auto set_slabs = [&](MoeGemmParams& p, int n, const uint8_t* q0, const uint8_t* b0, size_t bstride) {
+        for (int i = 0; i < n && i < MOE_MAX_SLABS; ++i) {
+            p.Q[i] = (const uint16_t*)(q0 + (size_t)i * qb);
+            p.LB[i] = (const uint16_t*)(b0 + (size_t)i * bstride);
+        }
+        p.nslab = n; p.q_slab_stride = (int64_t)(qb / 2); p.lb_slab_stride = (int64_t)(bstride / 2);
+    };
     // a rank of at most 16: the w2 GEMM's low-rank operand Q2 = h A2 comes out of the pair GEMM's epilogue as per-column-tile
-    // partials (h is not read again for it); two chunks take the separate pass over h
+    // partials (h is not read again for it); more chunks take separate passes over h
     const bool fuse_q2 = has_lora && rank <= 16;
     float* ccw = fuse_q2 ? (float*)ws.take(cc_bytes(R, f)) : nullptr;
     if (fuse_q2 && !ccw) return MOE_ERR_WORKSPACE;
     if (has_lora) {
         // lora order a1,b1,a3,b3,a2,b2; strides {expert, dim1, dim2}
         { TIMED("fwd.pack_lora");
-        MoePackBatch pb = {};
-        pb.E = E;
-        for (int c = 0; c < C; ++c) {
-            At1[c] = ws.take(pack_bytes(E, d)); At3[c] = ws.take(pack_bytes(E, d));
-            lb1[c] = ws.take(pack_bytes(E, f)); lb3[c] = ws.take(pack_bytes(E, f));
-            At2c[c] = ws.take(pack_bytes(E, f)); lb2[c] = ws.take(pack_bytes(E, d));
-            const int64_t r0 = 16 * c;
-            const int rk = (rank - 16 * c < 16) ? rank - 16 * c : 16;
-            auto L = [&](int i) { return (const uint16_t*)lora[i]; };
-            MoePackJob* j = pb.job + pb.njobs;
-            j[0] = {L(0) + r0 * ls[2], ls[0], ls[1], ls[2], (uint16_t*)At1[c], d, 1, rk};
-            j[1] = {L(1) + r0 * ls[4], ls[3], ls[5], ls[4], (uint16_t*)lb1[c], f, 0, rk};
-            j[2] = {L(2) + r0 * ls[8], ls[6], ls[7], ls[8], (uint16_t*)At3[c], d, 1, rk};
-            j[3] = {L(3) + r0 * ls[10], ls[9], ls[11], ls[10], (uint16_t*)lb3[c], f, 0, rk};
-            j[4] = {L(4) + r0 * ls[14], ls[12], ls[13], ls[14], (uint16_t*)At2c[c], f, 1, rk};
-            j[5] = {L(5) + r0 * ls[16], ls[15], ls[17], ls[16], (uint16_t*)lb2[c], d, 0, rk};
-            pb.njobs += 6;
-        }
-        pb.zero_ptr = (int*)skws; pb.zero_n = moe_gemm_num_counters();   // the K-split counters of the GEMMs below
-        TRY(moe_launch_pack_lora_batch(pb, st)); }
+        for (int c = 0; c < C; ++c) { At1[c] = ws.take(pbd); At3[c] = ws.take(pbd); At2c[c] = ws.take(pbf); }
+        lb13 = (uint8_t*)ws.take((size_t)2 * C * pbf);
+        lb2 = (uint8_t*)ws.take((size_t)C * pbd);
+        if (!lb13 || !lb2 || !At2c[C - 1]) return MOE_ERR_WORKSPACE;
+        for (int c0 = 0; c0 < C; c0 += 2) {   // six images per chunk, two chunks per launch
+            MoePackBatch pb = {};
+            pb.E = E;
+            for (int c = c0; c < C && c < c0 + 2; ++c) {
+                const int64_t r0 = 16 * c;
+                const int rk = (rank - 16 * c < 16) ? rank - 16 * c : 16;
+                auto L = [&](int i) { return (const uint16_t*)lora[i]; };
+                MoePackJob* j = pb.job + pb.njobs;
+                j[0] = {L(0) + r0 * ls[2], ls[0], ls[1], ls[2], (uint16_t*)At1[c], d, 1, rk};
+                j[1] = {L(1) + r0 * ls[4], ls[3], ls[5], ls[4], (uint16_t*)lb1(c), f, 0, rk};
+                j[2] = {L(2) + r0 * ls[8], ls[6], ls[7], ls[8], (uint16_t*)At3[c], d, 1, rk};
+                j[3] = {L(3) + r0 * ls[10], ls[9], ls[11], ls[10], (uint16_t*)lb3(c), f, 0, rk};
+                j[4] = {L(4) + r0 * ls[14], ls[12], ls[13], ls[14], (uint16_t*)At2c[c], f, 1, rk};
+                j[5] = {L(5) + r0 * ls[16], ls[15], ls[17], ls[16], (uint16_t*)lb2c(c), d, 0, rk};
+                pb.njobs += 6;
+            }
+            if (c0 == 0) { pb.zero_ptr = (int*)skws; pb.zero_n = moe_gemm_num_counters(); }   // the K-split counters of the GEMMs below
+            TRY(moe_launch_pack_lora_batch(pb, st));
+        } }
         { TIMED("fwd.rows_lora_x");
         for (int c = 0; c < C; ++c)
             TRY(moe_launch_rows_lora2(x, x, ldx, At1[c], At3[c], svp(0, c), svp(1, c), svp(3, c), svp(4, c), ldt, pos, pos64, offsets,
@@ -528,11 +549,8 @@ int moe_mlp_fwd(const void* x, int64_t ldx, const void* w1, const void* w3, cons
         p.X[0] = (const uint16_t*)x; p.ldx = ldx; p.nseg = 1;
         p.W[0] = (const uint16_t*)w1; p.W[1] = (const uint16_t*)w3; p.swe = f * d; p.ldw = d; p.nn = 0;
         if (has_lora) {   // gate slabs first, then up slabs
-            for (int c = 0; c < C; ++c) {
-                p.Q[c] = (const uint16_t*)svp(0, c); p.LB[c] = (const uint16_t*)lb1[c];
-                p.Q[C + c] = (const uint16_t*)svp(1, c); p.LB[C + c] = (const uint16_t*)lb3[c];
-            }
-            p.nslab = 2 * C; p.slab_mode = 1;
+            set_slabs(p, 2 * C, svp(0, 0), lb13, pbf);
+            p.slab_mode = 1;
         }
         p.Y[0] = (uint16_t*)h; p.Y[1] = (uint16_t*)gate; p.Y[2] = (uint16_t*)up; p.ldy = f;
         p.pos = pos; p.pos64 = pos64; p.offsets = offsets; p.off64 = off64;
@@ -552,16 +570,19 @@ int moe_mlp_fwd(const void* x, int64_t ldx, const void* w1, const void* w3, cons
         if (fuse_q2)   // the products over each column tile came out of the pair GEMM's epilogue: add the tiles, scale, round
             TRY(moe_launch_cc_reduce2(ccw, nullptr, (int)((f + 127) / 128), R, scaling, svp(2, 0), nullptr, svp(5, 0), nullptr, ldt, st, f16));
         else
-        TRY(moe_launch_rows_lora2(h, C > 1 ? h : nullptr, f, At2c[0], At2c[1], svp(2, 0), C > 1 ? svp(2, 1) : nullptr, svp(5, 0),
-                                  C > 1 ? svp(5, 1) : nullptr, ldt, nullptr, 0, offsets, off64, E, R, f, 1, 1, scaling, nullptr, st, nullptr, f16));
+        for (int c = 0; c < C; c += 2) {   // two chunks per launch: the twin's reads of h are served by L2
+            const bool two = c + 1 < C;
+            TRY(moe_launch_rows_lora2(h, two ? h : nullptr, f, At2c[c], two ? At2c[c + 1] : nullptr, svp(2, c), two ? svp(2, c + 1) : nullptr, svp(5, c),
+                                      two ? svp(5, c + 1) : nullptr, ldt, nullptr, 0, offsets, off64, E, R, f, 1, 1, scaling, nullptr, st, nullptr, f16));
+        }
     }
     {
         MoeGemmParams p = {};
         p.X[0] = (const uint16_t*)h; p.ldx = f; p.nseg = 1;
         p.W[0] = (const uint16_t*)w2; p.swe = f * d; p.ldw = d; p.nn = 1;
         if (has_lora) {
-            for (int c = 0; c < C; ++c) { p.Q[c] = (const uint16_t*)svp(2, c); p.LB[c] = (const uint16_t*)lb2[c]; }
-            p.nslab = C; p.slab_mode = 0;
+            set_slabs(p, C, svp(2, 0), lb2, pbd);
+            p.slab_mode = 0;
         }
         p.Y[0] = (uint16_t*)y; p.ldy = ldy;
         p.pos = pos; p.pos64 = pos64; p.offsets = offsets; p.off64 = off64;
@@ -596,19 +617,32 @@ int moe_mlp_bwd(const void* dy, int64_t lddy, int dy_grouped, int dy_fan_out, co
     const size_t qb = q_bytes(R);
     const int64_t ldt = pad_rows(R);
     const uint8_t* sv = (const uint8_t*)saved;
-    // adapters are worked through in C chunks of 16 rank columns (see moe_mlp_fwd); per chunk: packed factors and the
-    // interims P2, P1, P3, P2t, P1t, P3t
+    // adapters are worked through in C chunks of 16 rank columns (see moe_mlp_fwd): packed factors per chunk, and the
+    // interims in six groups of C blocks: P2, P1, P3, P2t, P1t, P3t
     const int C = has_lora ? (rank + 15) / 16 : 0;
-    void *bt2[2] = {}, *la2[2] = {}, *bt1[2] = {}, *bt3[2] = {}, *la1[2] = {}, *la3[2] = {};
+    const size_t pbd = pack_bytes(E, d), pbf = pack_bytes(E, f);
+    void *bt2[MLP_MAX_CHUNKS] = {}, *bt1[MLP_MAX_CHUNKS] = {}, *bt3[MLP_MAX_CHUNKS] = {};
+    uint8_t *la2 = nullptr, *la13 = nullptr;   // B-side images of the dh launch's slabs (a2 chunks) and of the dX launch's (a1 chunks, then a3 chunks)
+    auto la2c = [&](int c) { return la2 + (size_t)c * pbf; };
+    auto la1 = [&](int c) { return la13 + (size_t)c * pbd; };
+    auto la3 = [&](int c) { return la13 + (size_t)(C + c) * pbd; };
     uint8_t* pq = nullptr;
-    auto pqp = [&](int which, int c) { return pq + ((size_t)c * 6 + which) * qb; };   // which: 0 P2, 1 P1, 2 P3, 3 P2t, 4 P1t, 5 P3t
-    auto svp = [&](int which, int c) { return sv + ((size_t)c * 6 + which) * qb; };   // which: 0 Q1, 1 Q3, 2 Q2, 3 Qt1, 4 Qt3, 5 Qt2
+    auto pqp = [&](int which, int c) { return pq + ((size_t)which * C + c) * qb; };   // which: 0 P2, 1 P1, 2 P3, 3 P2t, 4 P1t, 5 P3t
+    auto svp = [&](int which, int c) { return sv + ((size_t)which * C + c) * qb; };   // which: 0 Q1, 1 Q3, 2 Q2, 3 Qt1, 4 Qt3, 5 Qt2
+    auto set_slabs = [&](MoeGemmParams& p, int n, const uint8_t* q0, const uint8_t* b0, size_t bstride) {
+        for (int i = 0; i < n && i < MOE_MAX_SLABS; ++i) {
+            p.Q[i] = (const uint16_t*)(q0 + (size_t)i * qb);
+            p.LB[i] = (const uint16_t*)(b0 + (size_t)i * bstride);
+        }
+        p.nslab = n; p.q_slab_stride = (int64_t)(qb / 2); p.lb_slab_stride = (int64_t)(bstride / 2);
+    };
+    auto chunk_rank = [&](int c) { return (rank - 16 * c < 16) ? rank - 16 * c : 16; };
     void* xw = nullptr;
     void* p2s = nullptr;
     float* ccw = nullptr;
     size_t xb = 0;
     // a rank of at most 16 (one chunk): the adapter gradients that sum over the rows of dgate, dup and h are produced by
-    // the dh GEMM's epilogue as per-row-tile partials; two chunks take the separate passes over those tensors
+    // the dh GEMM's epilogue as per-row-tile partials; more chunks take separate passes over those tensors
     const bool fuse_rc = has_lora && rank <= 16;
     if (!workspace || workspace_bytes < moe_mlp_workspace_bytes(R, E, d, f, has_lora ? rank : 0)) return MOE_ERR_WORKSPACE;
     Bump ws(workspace, workspace_bytes);
@@ -622,45 +656,51 @@ int moe_mlp_bwd(const void* dy, int64_t lddy, int dy_grouped, int dy_fan_out, co
         xb = 3 * moe_xtp_workspace_bytes(R, E, mx);   // paired reductions keep two sets of partials, the fused ones of the dh GEMM three
         xw = ws.take(xb);
         TIMED("bwd.pack_lora");
-        MoePackBatch pb = {};
-        pb.E = E;
         for (int c = 0; c < C; ++c) {
-            bt2[c] = ws.take(pack_bytes(E, d));  // fragment order of b2[e][r][n=d]
-            la1[c] = ws.take(pack_bytes(E, d));  // [e][n=d][r] = a1[e][n][r]
-            la3[c] = ws.take(pack_bytes(E, d));
-            la2[c] = ws.take(pack_bytes(E, f));  // [e][n=f][r] = a2[e][n][r]
-            bt1[c] = ws.take(pack_bytes(E, f));  // fragment order of b1[e][r][n=f]
-            bt3[c] = ws.take(pack_bytes(E, f));
-            const int64_t r0 = 16 * c;
-            const int rk = (rank - 16 * c < 16) ? rank - 16 * c : 16;
-            auto L = [&](int i) { return (const uint16_t*)lora[i]; };
-            MoePackJob* j = pb.job + pb.njobs;
-            j[0] = {L(5) + r0 * ls[16], ls[15], ls[17], ls[16], (uint16_t*)bt2[c], d, 1, rk};
-            j[1] = {L(4) + r0 * ls[14], ls[12], ls[13], ls[14], (uint16_t*)la2[c], f, 0, rk};
-            j[2] = {L(1) + r0 * ls[4], ls[3], ls[5], ls[4], (uint16_t*)bt1[c], f, 1, rk};
-            j[3] = {L(3) + r0 * ls[10], ls[9], ls[11], ls[10], (uint16_t*)bt3[c], f, 1, rk};
-            j[4] = {L(0) + r0 * ls[2], ls[0], ls[1], ls[2], (uint16_t*)la1[c], d, 0, rk};
-            j[5] = {L(2) + r0 * ls[8], ls[6], ls[7], ls[8], (uint16_t*)la3[c], d, 0, rk};
-            pb.njobs += 6;
+            bt2[c] = ws.take(pbd);  // fragment order of b2[e][r][n=d]
+            bt1[c] = ws.take(pbf);  // fragment order of b1[e][r][n=f]
+            bt3[c] = ws.take(pbf);
         }
-        if (!bt3[C - 1] || !xw) return MOE_ERR_WORKSPACE;
-        pb.zero_ptr = (int*)skws; pb.zero_n = moe_gemm_num_counters();   // the K-split counters of the GEMMs below
-        TRY(moe_launch_pack_lora_batch(pb, st));
+        la2 = (uint8_t*)ws.take((size_t)C * pbf);        // [e][n=f][r] = a2[e][n][r]
+        la13 = (uint8_t*)ws.take((size_t)2 * C * pbd);   // [e][n=d][r] = a1[e][n][r], a3 likewise
+        if (!la2 || !la13 || !bt3[C - 1] || !xw) return MOE_ERR_WORKSPACE;
+        for (int c0 = 0; c0 < C; c0 += 2) {   // six images per chunk, two chunks per launch
+            MoePackBatch pb = {};
+            pb.E = E;
+            for (int c = c0; c < C && c < c0 + 2; ++c) {
+                const int64_t r0 = 16 * c;
+                const int rk = chunk_rank(c);
+                auto L = [&](int i) { return (const uint16_t*)lora[i]; };
+                MoePackJob* j = pb.job + pb.njobs;
+                j[0] = {L(5) + r0 * ls[16], ls[15], ls[17], ls[16], (uint16_t*)bt2[c], d, 1, rk};
+                j[1] = {L(4) + r0 * ls[14], ls[12], ls[13], ls[14], (uint16_t*)la2c(c), f, 0, rk};
+                j[2] = {L(1) + r0 * ls[4], ls[3], ls[5], ls[4], (uint16_t*)bt1[c], f, 1, rk};
+                j[3] = {L(3) + r0 * ls[10], ls[9], ls[11], ls[10], (uint16_t*)bt3[c], f, 1, rk};
+                j[4] = {L(0) + r0 * ls[2], ls[0], ls[1], ls[2], (uint16_t*)la1(c), d, 0, rk};
+                j[5] = {L(2) + r0 * ls[8], ls[6], ls[7], ls[8], (uint16_t*)la3(c), d, 0, rk};
+                pb.njobs += 6;
+            }
+            if (c0 == 0) { pb.zero_ptr = (int*)skws; pb.zero_n = moe_gemm_num_counters(); }   // the K-split counters of the GEMMs below
+            TRY(moe_launch_pack_lora_batch(pb, st));
+        }
     }
     // ---- w2 backward: dh = (dy W2^T + P2 A2^T) * row_scale, SwiGLU backward in the epilogue
     if (has_lora) {
         TIMED("bwd.rows_lora_dy");
-        TRY(moe_launch_rows_lora2(dy, C > 1 ? dy : nullptr, lddy, bt2[0], bt2[1], pqp(0, 0), C > 1 ? pqp(0, 1) : nullptr, pqp(3, 0),
-                                  C > 1 ? pqp(3, 1) : nullptr, ldt, pos, pos64, offsets, off64, E, R, d, dy_fan_out, dy_grouped, scaling,
-                                  row_scale, st, p2s, f16));
+        for (int c = 0; c < C; c += 2) {
+            const bool two = c + 1 < C;
+            TRY(moe_launch_rows_lora2(dy, two ? dy : nullptr, lddy, bt2[c], two ? bt2[c + 1] : nullptr, pqp(0, c), two ? pqp(0, c + 1) : nullptr, pqp(3, c),
+                                      two ? pqp(3, c + 1) : nullptr, ldt, pos, pos64, offsets, off64, E, R, d, dy_fan_out, dy_grouped, scaling,
+                                      row_scale, st, p2s, f16));
+        }
     }
     {
         MoeGemmParams p = {};
         p.X[0] = (const uint16_t*)dy; p.ldx = lddy; p.nseg = 1;
         p.W[0] = (const uint16_t*)w2; p.swe = f * d; p.ldw = d; p.nn = 0;  // (E, K=d, N=f): n rows, k contiguous
         if (has_lora) {
-            for (int c = 0; c < C; ++c) { p.Q[c] = (const uint16_t*)pqp(0, c); p.LB[c] = (const uint16_t*)la2[c]; }
-            p.nslab = C; p.slab_mode = 0;
+            set_slabs(p, C, pqp(0, 0), la2, pbf);
+            p.slab_mode = 0;
         }
         p.Y[0] = (uint16_t*)dgate; p.Y[1] = (uint16_t*)dup; p.ldy = f;
         p.H1 = (const uint16_t*)gate; p.H3 = (const uint16_t*)up; p.ldh = f; p.row_scale = row_scale;
@@ -698,34 +738,39 @@ int moe_mlp_bwd(const void* dy, int64_t lddy, int dy_grouped, int dy_fan_out, co
             TRY(moe_launch_xtp_reduce2(part, part + one / sizeof(float), lg[1], lg[3], sb1, sb3, rank, rank, offsets, off64, E, f, 1.f, st, f16));
             TRY(moe_launch_xtp_reduce2(part + 2 * (one / sizeof(float)), nullptr, dA2, nullptr, sa2, nullptr, rank, 0, offsets, off64, E, f, 1.f, st, f16));
         } else
-        TRY(moe_launch_xtp2(h, C > 1 ? h : nullptr, f, nullptr, 0, 1, pqp(3, 0), C > 1 ? pqp(3, 1) : nullptr, ldt, nullptr, dA2,
-                            C > 1 ? dA2 + 16 * gs[14] : nullptr, sa2, sa2, rank < 16 ? rank : 16, C > 1 ? rank - 16 : 0, offsets, off64, E, R, f,
-                            1.f, xw, xb, st, f16));
-        TRY(moe_launch_xtp2(dy, C > 1 ? dy : nullptr, lddy, dy_grouped ? nullptr : pos, pos64, dy_fan_out, svp(5, 0),
-                            C > 1 ? svp(5, 1) : nullptr, ldt, row_scale, dB2, C > 1 ? dB2 + 16 * gs[16] : nullptr, sb2, sb2,
-                            rank < 16 ? rank : 16, C > 1 ? rank - 16 : 0, offsets, off64, E, R, d, 1.f, xw, xb, st, f16)); }
+        for (int c = 0; c < C; c += 2) {   // two chunks per launch: the twin's reads of h are served by L2
+            const bool two = c + 1 < C;
+            TRY(moe_launch_xtp2(h, two ? h : nullptr, f, nullptr, 0, 1, pqp(3, c), two ? pqp(3, c + 1) : nullptr, ldt, nullptr, dA2 + 16 * c * gs[14],
+                                two ? dA2 + 16 * (c + 1) * gs[14] : nullptr, sa2, sa2, chunk_rank(c), two ? chunk_rank(c + 1) : 0, offsets, off64, E, R, f,
+                                1.f, xw, xb, st, f16));
+        }
+        for (int c = 0; c < C; c += 2) {
+            const bool two = c + 1 < C;
+            TRY(moe_launch_xtp2(dy, two ? dy : nullptr, lddy, dy_grouped ? nullptr : pos, pos64, dy_fan_out, svp(5, c),
+                                two ? svp(5, c + 1) : nullptr, ldt, row_scale, dB2 + 16 * c * gs[16], two ? dB2 + 16 * (c + 1) * gs[16] : nullptr, sb2, sb2,
+                                chunk_rank(c), two ? chunk_rank(c + 1) : 0, offsets, off64, E, R, d, 1.f, xw, xb, st, f16));
+        } }
         // ---- w1 / w3 backward
         TIMED("bwd.rows_lora_dgate_dup");
         if (fuse_rc) {   // the products over each column tile came out of the dh GEMM's epilogue: add the tiles, scale, round
             const size_t cone = cc_bytes(R, f) / 2 / sizeof(float);
             TRY(moe_launch_cc_reduce2(ccw, ccw + cone, (int)((f + 255) / 256), R, scaling, pqp(1, 0), pqp(2, 0), pqp(4, 0), pqp(5, 0), ldt, st, f16));
-        } else {   // two chunks: the chunks of one adapter share a launch, so that dgate and dup are each read once
-            TRY(moe_launch_rows_lora2(dgate, dgate, f, bt1[0], bt1[1], pqp(1, 0), pqp(1, 1), pqp(4, 0), pqp(4, 1), ldt, nullptr, 0, offsets,
-                                      off64, E, R, f, 1, 1, scaling, nullptr, st, nullptr, f16));
-            TRY(moe_launch_rows_lora2(dup, dup, f, bt3[0], bt3[1], pqp(2, 0), pqp(2, 1), pqp(5, 0), pqp(5, 1), ldt, nullptr, 0, offsets,
-                                      off64, E, R, f, 1, 1, scaling, nullptr, st, nullptr, f16));
+        } else
+        for (int c = 0; c < C; c += 2) {   // two chunks of one adapter per launch, so that dgate and dup are each fetched once per pair of chunks
+            const bool two = c + 1 < C;
+            TRY(moe_launch_rows_lora2(dgate, two ? dgate : nullptr, f, bt1[c], two ? bt1[c + 1] : nullptr, pqp(1, c), two ? pqp(1, c + 1) : nullptr, pqp(4, c),
+                                      two ? pqp(4, c + 1) : nullptr, ldt, nullptr, 0, offsets, off64, E, R, f, 1, 1, scaling, nullptr, st, nullptr, f16));
+            TRY(moe_launch_rows_lora2(dup, two ? dup : nullptr, f, bt3[c], two ? bt3[c + 1] : nullptr, pqp(2, c), two ? pqp(2, c + 1) : nullptr, pqp(5, c),
+                                      two ? pqp(5, c + 1) : nullptr, ldt, nullptr, 0, offsets, off64, E, R, f, 1, 1, scaling, nullptr, st, nullptr, f16));
         }
     }
     {
         MoeGemmParams p = {};
         p.X[0] = (const uint16_t*)dgate; p.X[1] = (const uint16_t*)dup; p.ldx = f; p.nseg = 2;
         p.W[0] = (const uint16_t*)w1; p.W[1] = (const uint16_t*)w3; p.swe = f * d; p.ldw = d; p.nn = 1;  // (E, K=f, N=d)
-        if (has_lora) {
-            for (int c = 0; c < C; ++c) {
-                p.Q[c] = (const uint16_t*)pqp(1, c); p.LB[c] = (const uint16_t*)la1[c];
-                p.Q[C + c] = (const uint16_t*)pqp(2, c); p.LB[C + c] = (const uint16_t*)la3[c];
-            }
-            p.nslab = 2 * C; p.slab_mode = 0;
+        if (has_lora) {   // P1 chunks, then P3 chunks; every slab feeds every column
+            set_slabs(p, 2 * C, pqp(1, 0), la13, pbd);
+            p.slab_mode = 0;
         }
         p.Y[0] = (uint16_t*)dx_rows; p.ldy = lddx;
         p.pos = pos; p.pos64 = pos64; p.offsets = offsets; p.off64 = off64;
@@ -742,15 +787,18 @@ int moe_mlp_bwd(const void* dy, int64_t lddy, int dy_grouped, int dy_fan_out, co
         const int64_t sa1[3] = {gs[0], gs[1], gs[2]}, sa3[3] = {gs[6], gs[7], gs[8]};
         const int64_t sb1[3] = {gs[3], gs[5], gs[4]}, sb3[3] = {gs[9], gs[11], gs[10]};
         for (int c = 0; c < C; ++c) {
-            const int rk = (rank - 16 * c < 16) ? rank - 16 * c : 16;
+            const int rk = chunk_rank(c);
             TRY(moe_launch_xtp2(x, x, ldx, pos, pos64, fan_out, pqp(4, c), pqp(5, c), ldt, nullptr, (uint16_t*)lg[0] + 16 * c * gs[2],
                                 (uint16_t*)lg[2] + 16 * c * gs[8], sa1, sa3, rk, rk, offsets, off64, E, R, d, 1.f, xw, xb, st, f16));
         }
-        if (!fuse_rc) {   // two chunks: the chunks of one adapter share a launch, so that dgate and dup are each read once
-            TRY(moe_launch_xtp2(dgate, dgate, f, nullptr, 0, 1, svp(3, 0), svp(3, 1), ldt, nullptr, lg[1], (uint16_t*)lg[1] + 16 * gs[4],
-                                sb1, sb1, 16, rank - 16, offsets, off64, E, R, f, 1.f, xw, xb, st, f16));
-            TRY(moe_launch_xtp2(dup, dup, f, nullptr, 0, 1, svp(4, 0), svp(4, 1), ldt, nullptr, lg[3], (uint16_t*)lg[3] + 16 * gs[10],
-                                sb3, sb3, 16, rank - 16, offsets, off64, E, R, f, 1.f, xw, xb, st, f16));
+        if (!fuse_rc)
+        for (int c = 0; c < C; c += 2) {   // two chunks of one adapter per launch, so that dgate and dup are each fetched once per pair of chunks
+            const bool two = c + 1 < C;
+            const int rk0 = chunk_rank(c), rk1 = two ? chunk_rank(c + 1) : 0;
+            TRY(moe_launch_xtp2(dgate, two ? dgate : nullptr, f, nullptr, 0, 1, svp(3, c), two ? svp(3, c + 1) : nullptr, ldt, nullptr, (uint16_t*)lg[1] + 16 * c * gs[4],
+                                two ? (uint16_t*)lg[1] + 16 * (c + 1) * gs[4] : nullptr, sb1, sb1, rk0, rk1, offsets, off64, E, R, f, 1.f, xw, xb, st, f16));
+            TRY(moe_launch_xtp2(dup, two ? dup : nullptr, f, nullptr, 0, 1, svp(4, c), two ? svp(4, c + 1) : nullptr, ldt, nullptr, (uint16_t*)lg[3] + 16 * c * gs[10],
+                                two ? (uint16_t*)lg[3] + 16 * (c + 1) * gs[10] : nullptr, sb3, sb3, rk0, rk1, offsets, off64, E, R, f, 1.f, xw, xb, st, f16));
         }
     }
     return MOE_OK;

@@ -68,7 +68,7 @@ def _fast_path_ok(x, w1, w2, w3, lora: Optional[LoraViews]) -> bool:
         return False
     if not (w1.is_contiguous() and w2.is_contiguous() and w3.is_contiguous()):
         return False
-    if lora is not None and lora.a1.size(2) > 32:   # the fused launches take an adapter as one or two 16-wide rank chunks
+    if lora is not None and lora.a1.size(2) > 128:   # the fused launches take an adapter as up to eight 16-wide rank chunks
         return False
     # gathered activation rows and one expert's matrix are addressed with 32-bit byte offsets (the same check the library
     # makes before it enqueues anything); the number of rows is otherwise not limited
@@ -205,7 +205,7 @@ def fused_expert_mlp(x, w1, w2, w3, k, sorted_scattered_idxs, expert_offsets, lo
     require_gpu(x, w1, w2, w3, sorted_scattered_idxs, expert_offsets)
     lt = (None,) * 6 if lora is None else tuple(lora)
     if not _fast_path_ok(x, w1, w2, w3, lora):
-        raise RuntimeError("fused_expert_mlp needs bf16, contiguous (E,f,d) weights, d and f multiples of 64 and rank <= 32; "
+        raise RuntimeError("fused_expert_mlp needs bf16, contiguous (E,f,d) weights, d and f multiples of 64 and rank <= 128; "
                            "use scattermoe_permute_and_compute for other cases")
     return FusedExpertMLP.apply(x, w1, w3, w2, *lt, lora_alpha, gates, sorted_scattered_idxs.contiguous(),
                                 expert_offsets.contiguous(), k, grouped_out)
