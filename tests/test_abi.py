@@ -81,3 +81,24 @@ def test_size_limits_are_checked_before_anything_is_enqueued():
     # many rows alone are fine: the call gets as far as the workspace check (status -3), i.e. past the size checks
     assert fwd(2 * 200000, 4096, 14336, 2) == -3
     assert lib.moe_mlp_workspace_bytes(400000, 8, 4096, 14336, 16) > 0
+
+
+def test_fused_layer_rank_limit_is_checked_on_the_host():
+    """The fused layer takes an adapter as up to eight chunks of 16 rank columns: rank 128 gets past the shape checks (as
+    far as the workspace check), rank 129 is refused with MOE_ERR_UNSUPPORTED before anything is enqueued; the sizes of
+    the saved interims and of the workspace grow with the number of chunks."""
+    import ctypes
+    from moe_distributed_training_amd._lib import lib
+    one = 16   # non-null, 16-byte aligned stand-ins: never dereferenced
+    lora = (ctypes.c_void_p * 6)(*([one] * 6))
+    strides = (ctypes.c_int64 * 18)(*([1] * 18))
+
+    def fwd(rank):
+        return lib.moe_mlp_fwd(one, 4096, one, one, one, lora, strides, rank, 1.0, one, one, one, one, 4096, one, 0, one, 0,
+                               8, 8192, 4096, 14336, 2, 0, 0, one, None, 0, None)
+    assert fwd(128) == -3 and fwd(72) == -3 and fwd(16) == -3
+    assert fwd(129) == -2 and fwd(256) == -2
+    saved = [lib.moe_mlp_saved_bytes(8192, r) for r in (16, 17, 32, 33, 128)]
+    assert saved[1] == saved[2] == 2 * saved[0] and saved[3] == 3 * saved[0] and saved[4] == 8 * saved[0]
+    ws = [lib.moe_mlp_workspace_bytes(8192, 8, 4096, 14336, r) for r in (0, 16, 32, 64, 128)]
+    assert ws == sorted(ws) and len(set(ws)) == 5
