@@ -473,6 +473,7 @@ int moe_launch_rows_lora2(const void* X, const void* X2, int64_t ldx, const void
     const RowsLoraJob j1 = {(const uint16_t*)X2, (const uint16_t*)At2, (uint16_t*)Q2, (uint16_t*)Qt2, nullptr};
     // 32-row tiles halve the adapter traffic, but two workgroups fit a compute unit: use them when the launch has
     // about that many, otherwise 16-row tiles (three fit)
+    if ((R / 16 + E) * 2 + 16 >= ((int64_t)1 << 31)) return MOE_ERR_UNSUPPORTED;   // workgroups of the launch, as a 32-bit grid size
     const int cus = moe_device_cus();
     const int64_t tiles32 = (R / 32 + E) * (two ? 2 : 1);
     if (tiles32 >= 3 * (int64_t)cus / 2) {
